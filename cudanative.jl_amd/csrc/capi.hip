@@ -1,0 +1,633 @@
+// C ABI of libmiwmma.so (declared in include/miwmma.h): argument validation,
+// error reporting, memory / stream / event plumbing and kernel dispatch.
+// Nothing here falls back to the CPU: without a usable HIP device every entry
+// that needs one returns the HIP error.
+#include "../../include/miwmma.h"
+#include "kernels.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char *what)
+{
+    // Clear the sticky "last error" so that it is not reported by a later call.
+    (void)hipGetLastError();
+    return fail((int)e, "%s: %s (%s)", what, hipGetErrorString(e), hipGetErrorName(e));
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e_ = (expr);                         \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+bool valid_layout(int l) { return l == MIW_ROW_MAJOR || l == MIW_COL_MAJOR; }
+bool valid_dtype(int t) { return t == MIW_F16 || t == MIW_F32; }
+bool valid_as(int a) { return a == MIW_AS_GENERIC || a == MIW_AS_GLOBAL || a == MIW_AS_SHARED; }
+size_t dtype_size(int t) { return t == MIW_F16 ? 2 : 4; }
+
+int check_shape(int m, int n, int k)
+{
+    if (m != 16 || n != 16 || k != 16)
+        return fail(MIW_ERR_INVALID_SHAPE, "Invalid shape for WMMA: (M, N, K) = (%d, %d, %d)", m, n, k);
+    return 0;
+}
+
+hipStream_t as_stream(void *s) { return (hipStream_t)s; }
+
+struct named_kernel {
+    std::string name;
+    const void *fn;
+};
+
+std::vector<named_kernel> &registry()
+{
+    static std::vector<named_kernel> r = [] {
+        std::vector<named_kernel> v;
+        for (int i = 0; i < miw::frag_kernel_count(); i++) {
+            const char *n = miw::frag_kernel_name(i);
+            v.push_back({n, miw::frag_kernel_symbol(n)});
+        }
+        for (int i = 0; i < miw::tiled_variant_count(); i++)
+            v.push_back({std::string("gemm_") + miw::tiled_variant_at(i).name, miw::tiled_kernel_symbol(i)});
+        return v;
+    }();
+    return r;
+}
+
+// Fill defaults and validate a GEMM descriptor; on success writes kernel params.
+int resolve_gemm(const miw_gemm_desc *d, const void *A, const void *B, const void *C, void *D, miw::gemm_params *out,
+                 bool *f16acc)
+{
+    if (!d) return fail(MIW_ERR_NULL_POINTER, "gemm: null descriptor");
+    if (!valid_layout(d->a_layout) || !valid_layout(d->b_layout) || !valid_layout(d->c_layout) ||
+        !valid_layout(d->d_layout))
+        return fail(MIW_ERR_INVALID_LAYOUT, "Invalid layout for WMMA: a=%d b=%d c=%d d=%d", d->a_layout, d->b_layout,
+                    d->c_layout, d->d_layout);
+    if (!valid_dtype(d->c_type) || !valid_dtype(d->d_type) || !valid_dtype(d->acc_type))
+        return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: c=%d d=%d acc=%d", d->c_type, d->d_type,
+                    d->acc_type);
+    if (d->m <= 0 || d->n <= 0 || d->k <= 0 || d->m % 16 || d->n % 16 || d->k % 16)
+        return fail(MIW_ERR_INVALID_SHAPE, "gemm: M, N, K must be positive multiples of 16, got (%lld, %lld, %lld)",
+                    (long long)d->m, (long long)d->n, (long long)d->k);
+    if (d->m > (1ll << 30) || d->n > (1ll << 30) || d->k > (1ll << 30))
+        return fail(MIW_ERR_INVALID_SHAPE, "gemm: dimension too large");
+    if (d->batch < 1 || d->batch > 65535)
+        return fail(MIW_ERR_INVALID_VALUE, "gemm: batch must be in 1..65535, got %lld", (long long)d->batch);
+    *f16acc = d->acc_type == MIW_F16;
+    if (*f16acc && (d->c_type != MIW_F16 || d->d_type != MIW_F16))
+        return fail(MIW_ERR_INVALID_TYPE, "gemm: Float16 accumulation needs Float16 C and D");
+    if (!A || !B || !D || (d->use_c && !C)) return fail(MIW_ERR_NULL_POINTER, "gemm: null operand pointer");
+
+    miw::gemm_params p{};
+    p.A = (const _Float16 *)A;
+    p.B = (const _Float16 *)B;
+    p.C = C;
+    p.D = D;
+    p.M = d->m; p.N = d->n; p.K = d->k;
+    p.a_row = d->a_layout == MIW_ROW_MAJOR;
+    p.b_row = d->b_layout == MIW_ROW_MAJOR;
+    p.c_row = d->c_layout == MIW_ROW_MAJOR;
+    p.d_row = d->d_layout == MIW_ROW_MAJOR;
+    const long mina = p.a_row ? p.K : p.M, minb = p.b_row ? p.N : p.K;
+    const long minc = p.c_row ? p.N : p.M, mind = p.d_row ? p.N : p.M;
+    p.lda = d->lda ? d->lda : mina;
+    p.ldb = d->ldb ? d->ldb : minb;
+    p.ldc = d->ldc ? d->ldc : minc;
+    p.ldd = d->ldd ? d->ldd : mind;
+    if (p.lda < mina || p.ldb < minb || p.ldd < mind || (d->use_c && p.ldc < minc))
+        return fail(MIW_ERR_INVALID_VALUE, "gemm: leading dimension smaller than the matrix extent");
+    p.sa = d->stride_a ? d->stride_a : p.lda * (p.a_row ? p.M : p.K);
+    p.sb = d->stride_b ? d->stride_b : p.ldb * (p.b_row ? p.K : p.N);
+    p.sc = d->stride_c ? d->stride_c : p.ldc * (p.c_row ? p.M : p.N);
+    p.sd = d->stride_d ? d->stride_d : p.ldd * (p.d_row ? p.M : p.N);
+    p.batch = d->batch;
+    p.use_c = d->use_c != 0;
+    p.alpha = d->alpha;
+    p.beta = d->beta;
+    if (((uintptr_t)A & 1) || ((uintptr_t)B & 1) || ((uintptr_t)D & (dtype_size(d->d_type) - 1)) ||
+        (p.use_c && ((uintptr_t)C & (dtype_size(d->c_type) - 1))))
+        return fail(MIW_ERR_MISALIGNED, "gemm: operand pointer not aligned to its element type");
+    *out = p;
+    return 0;
+}
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// Can tiled variant i (0-based) run this problem?
+bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
+{
+    const miw::tiled_variant &v = miw::tiled_variant_at(i);
+    // In canonical terms bm tiles the contiguous dimension of D.
+    const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
+    if (I % v.bm || J % v.bn || p.K % v.bk) return false;
+    if (!aligned16(p.A) || !aligned16(p.B) || !aligned16(p.D) || (p.use_c && !aligned16(p.C))) return false;
+    if (p.lda % 8 || p.ldb % 8 || p.sa % 8 || p.sb % 8) return false;
+    const long cper = 16 / (long)dtype_size(c_type), dper = 16 / (long)dtype_size(d_type);
+    if (p.ldd % dper || p.sd % dper) return false;
+    if (p.use_c && (p.ldc % cper || p.sc % cper)) return false;
+    // 32-bit offsets inside one operand tile
+    if (p.lda * 256 >= (1l << 31) || p.ldb * 256 >= (1l << 31)) return false;
+    if (f16acc && (p.alpha != 1.0f || (acc_chunk != 0 && acc_chunk != miw::tiled_f16acc_chunk()))) return false;
+    return true;
+}
+
+int g_cu_count = 0;
+
+int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
+{
+    // Largest tile that still gives every CU a workgroup; else the one with most workgroups.
+    const int cus = g_cu_count > 0 ? g_cu_count : 256;
+    const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
+    int best = -1;
+    long best_wgs = -1;
+    for (int i = 0; i < miw::tiled_variant_count(); i++) {
+        if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk)) continue;
+        const miw::tiled_variant &v = miw::tiled_variant_at(i);
+        const long wgs = (I / v.bm) * (J / v.bn) * p.batch;
+        if (wgs >= cus) return i + 1;
+        if (wgs > best_wgs) { best = i; best_wgs = wgs; }
+    }
+    if (best >= 0) return best + 1;
+    return miw::tiled_variant_count() + 1;  // fragment-op kernel
+}
+
+int run_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, hipStream_t s)
+{
+    const int nt = miw::tiled_variant_count();
+    int variant = d->variant;
+    if (variant < 0 || variant > nt + 1) return fail(MIW_ERR_INVALID_VALUE, "gemm: unknown variant %d", variant);
+    if (variant == 0) variant = pick_variant(p, d->c_type, d->d_type, f16acc, d->acc_chunk);
+    if (variant == nt + 1) {
+        if (f16acc && d->acc_chunk != 0 && d->acc_chunk != 16)
+            return fail(MIW_ERR_UNSUPPORTED, "gemm: the fragment-op kernel rounds every 16 k-values (acc_chunk %d asked)",
+                        d->acc_chunk);
+        HIP_TRY(miw::launch_gemm_fragops(p, d->c_type, d->d_type, f16acc, s));
+        return 0;
+    }
+    if (!tiled_fits(variant - 1, p, d->c_type, d->d_type, f16acc, d->acc_chunk))
+        return fail(MIW_ERR_UNSUPPORTED,
+                    "gemm: variant %d (%s) needs tile-divisible sizes, 16-byte aligned operands and leading "
+                    "dimensions%s",
+                    variant, miw::tiled_variant_at(variant - 1).name,
+                    f16acc ? ", alpha == 1 and its own acc_chunk" : "");
+    HIP_TRY(miw::launch_gemm_tiled(variant - 1, p, d->c_type, d->d_type, f16acc, s));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *miw_last_error(void) { return g_err; }
+
+int miw_init(int device)
+{
+    int n = 0;
+    HIP_TRY(hipGetDeviceCount(&n));
+    if (device < 0 || device >= n) return fail(MIW_ERR_INVALID_VALUE, "init: device %d out of range (count %d)", device, n);
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(MIW_ERR_UNSUPPORTED, "init: kernels are built for gfx950, device is %s", prop.gcnArchName);
+    g_cu_count = prop.multiProcessorCount;
+    g_err[0] = 0;
+    return 0;
+}
+
+int miw_device_info_get(miw_device_info *out)
+{
+    if (!out) return fail(MIW_ERR_NULL_POINTER, "device_info: null output");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    memset(out, 0, sizeof(*out));
+    snprintf(out->name, sizeof(out->name), "%s", prop.name);
+    snprintf(out->arch, sizeof(out->arch), "%s", prop.gcnArchName);
+    out->cu_count = prop.multiProcessorCount;
+    out->wave_size = prop.warpSize;
+    out->clock_mhz = prop.clockRate / 1000;
+    out->mem_clock_mhz = prop.memoryClockRate / 1000;
+    out->mem_bus_bits = prop.memoryBusWidth;
+    out->l2_bytes = prop.l2CacheSize;
+    out->max_threads_per_block = prop.maxThreadsPerBlock;
+    out->lds_per_block = prop.sharedMemPerBlock;
+    out->hbm_bytes = prop.totalGlobalMem;
+    out->peak_f16_tflops = (double)out->cu_count * 4.0 * 1024.0 * (double)out->clock_mhz * 1e6 / 1e12;
+    return 0;
+}
+
+int miw_malloc(void **out, size_t bytes)
+{
+    if (!out) return fail(MIW_ERR_NULL_POINTER, "malloc: null output");
+    *out = nullptr;
+    if (bytes == 0) return 0;
+    HIP_TRY(hipMalloc(out, bytes));
+    return 0;
+}
+
+int miw_free(void *p)
+{
+    if (!p) return 0;
+    HIP_TRY(hipFree(p));
+    return 0;
+}
+
+int miw_memcpy_h2d(void *dst, const void *src, size_t bytes)
+{
+    if (bytes == 0) return 0;
+    if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "memcpy_h2d: null pointer");
+    HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int miw_memcpy_d2h(void *dst, const void *src, size_t bytes)
+{
+    if (bytes == 0) return 0;
+    if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "memcpy_d2h: null pointer");
+    HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int miw_memcpy_d2d(void *dst, const void *src, size_t bytes)
+{
+    if (bytes == 0) return 0;
+    if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "memcpy_d2d: null pointer");
+    HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice));
+    return 0;
+}
+
+int miw_memset(void *dst, int byte, size_t bytes)
+{
+    if (bytes == 0) return 0;
+    if (!dst) return fail(MIW_ERR_NULL_POINTER, "memset: null pointer");
+    HIP_TRY(hipMemset(dst, byte, bytes));
+    return 0;
+}
+
+int miw_stream_create(void **out)
+{
+    if (!out) return fail(MIW_ERR_NULL_POINTER, "stream_create: null output");
+    hipStream_t s;
+    HIP_TRY(hipStreamCreate(&s));  // default priority only
+    *out = (void *)s;
+    return 0;
+}
+
+int miw_stream_destroy(void *stream)
+{
+    if (!stream) return 0;
+    HIP_TRY(hipStreamDestroy(as_stream(stream)));
+    return 0;
+}
+
+int miw_sync(void *stream)
+{
+    if (stream) HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    else HIP_TRY(hipDeviceSynchronize());
+    return 0;
+}
+
+int miw_event_create(void **out)
+{
+    if (!out) return fail(MIW_ERR_NULL_POINTER, "event_create: null output");
+    hipEvent_t e;
+    HIP_TRY(hipEventCreate(&e));
+    *out = (void *)e;
+    return 0;
+}
+
+int miw_event_destroy(void *event)
+{
+    if (!event) return 0;
+    HIP_TRY(hipEventDestroy((hipEvent_t)event));
+    return 0;
+}
+
+int miw_event_record(void *event, void *stream)
+{
+    if (!event) return fail(MIW_ERR_NULL_POINTER, "event_record: null event");
+    HIP_TRY(hipEventRecord((hipEvent_t)event, as_stream(stream)));
+    return 0;
+}
+
+int miw_event_synchronize(void *event)
+{
+    if (!event) return fail(MIW_ERR_NULL_POINTER, "event_synchronize: null event");
+    HIP_TRY(hipEventSynchronize((hipEvent_t)event));
+    return 0;
+}
+
+int miw_event_elapsed_ms(float *ms, void *start, void *stop)
+{
+    if (!ms || !start || !stop) return fail(MIW_ERR_NULL_POINTER, "event_elapsed_ms: null argument");
+    HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return 0;
+}
+
+// ------------------------------------------------------------- fragments ---
+
+int miw_frag_elems_per_lane(int use, int dtype)
+{
+    if (use < MIW_MATRIX_A || use > MIW_ACCUMULATOR) return fail(MIW_ERR_INVALID_VALUE, "Invalid fragment use %d", use);
+    if (!valid_dtype(dtype)) return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: %d", dtype);
+    if (use != MIW_ACCUMULATOR && dtype != MIW_F16)
+        return fail(MIW_ERR_INVALID_TYPE, "Invalid type Float32 for matrix %s", use == MIW_MATRIX_A ? "a" : "b");
+    return 4;
+}
+
+size_t miw_frag_image_bytes(int use, int dtype)
+{
+    int n = miw_frag_elems_per_lane(use, dtype);
+    return n > 0 ? (size_t)n * 64 * dtype_size(dtype) : 0;
+}
+
+int miw_frag_load(int use, int dtype, int layout, int addr_space, int m, int n, int k, const void *addr,
+                  int64_t stride, void *frag, void *stream)
+{
+    if (int rc = check_shape(m, n, k)) return rc;
+    if (!valid_as(addr_space)) return fail(MIW_ERR_INVALID_AS, "Invalid address space for WMMA: %d", addr_space);
+    if (!valid_layout(layout)) return fail(MIW_ERR_INVALID_LAYOUT, "Invalid layout for WMMA: %d", layout);
+    if (int ne = miw_frag_elems_per_lane(use, dtype); ne < 0) return ne;
+    if (!addr || !frag) return fail(MIW_ERR_NULL_POINTER, "frag_load: null pointer");
+    if (stride < 16) return fail(MIW_ERR_INVALID_VALUE, "frag_load: stride %lld smaller than the tile", (long long)stride);
+    if ((uintptr_t)addr & (dtype_size(dtype) - 1)) return fail(MIW_ERR_MISALIGNED, "frag_load: misaligned address");
+    HIP_TRY(miw::launch_frag_load(use, dtype, layout == MIW_ROW_MAJOR, addr_space, addr, (long)stride, frag,
+                                  as_stream(stream)));
+    return 0;
+}
+
+int miw_frag_store(int dtype, int layout, int addr_space, int m, int n, int k, void *addr, const void *frag,
+                   int64_t stride, void *stream)
+{
+    if (int rc = check_shape(m, n, k)) return rc;
+    if (!valid_as(addr_space)) return fail(MIW_ERR_INVALID_AS, "Invalid address space for WMMA: %d", addr_space);
+    if (!valid_layout(layout)) return fail(MIW_ERR_INVALID_LAYOUT, "Invalid layout for WMMA: %d", layout);
+    if (!valid_dtype(dtype)) return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: %d", dtype);
+    if (!addr || !frag) return fail(MIW_ERR_NULL_POINTER, "frag_store: null pointer");
+    if (stride < 16) return fail(MIW_ERR_INVALID_VALUE, "frag_store: stride %lld smaller than the tile", (long long)stride);
+    if ((uintptr_t)addr & (dtype_size(dtype) - 1)) return fail(MIW_ERR_MISALIGNED, "frag_store: misaligned address");
+    HIP_TRY(miw::launch_frag_store(dtype, layout == MIW_ROW_MAJOR, addr_space, addr, frag, (long)stride,
+                                   as_stream(stream)));
+    return 0;
+}
+
+int miw_frag_fill(int dtype, float value, void *frag, void *stream)
+{
+    if (!valid_dtype(dtype)) return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: %d", dtype);
+    if (!frag) return fail(MIW_ERR_NULL_POINTER, "frag_fill: null pointer");
+    HIP_TRY(miw::launch_frag_fill(dtype, value, frag, as_stream(stream)));
+    return 0;
+}
+
+int miw_frag_map(int dtype, int op, float scalar, const void *in, void *out, size_t n_elems, void *stream)
+{
+    if (!valid_dtype(dtype)) return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: %d", dtype);
+    if (op != MIW_OP_MUL && op != MIW_OP_ADD) return fail(MIW_ERR_INVALID_VALUE, "frag_map: unknown operator %d", op);
+    if (n_elems && (!in || !out)) return fail(MIW_ERR_NULL_POINTER, "frag_map: null pointer");
+    HIP_TRY(miw::launch_frag_map(dtype, op, scalar, in, out, n_elems, as_stream(stream)));
+    return 0;
+}
+
+int miw_frag_mma(int a_layout, int b_layout, int c_type, int d_type, const void *a_frag, const void *b_frag,
+                 const void *c_frag, void *d_frag, void *stream)
+{
+    if (!valid_layout(a_layout) || !valid_layout(b_layout))
+        return fail(MIW_ERR_INVALID_LAYOUT, "Invalid layout for WMMA: a=%d b=%d", a_layout, b_layout);
+    if (!valid_dtype(c_type) || !valid_dtype(d_type))
+        return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: c=%d d=%d", c_type, d_type);
+    if (!a_frag || !b_frag || !c_frag || !d_frag) return fail(MIW_ERR_NULL_POINTER, "frag_mma: null pointer");
+    HIP_TRY(miw::launch_frag_mma(c_type, d_type, a_frag, b_frag, c_frag, d_frag, as_stream(stream)));
+    return 0;
+}
+
+int miw_wmma_mac(const miw_mac_desc *d, const void *A, const void *B, const void *C, void *D, void *stream)
+{
+    if (!d) return fail(MIW_ERR_NULL_POINTER, "wmma_mac: null descriptor");
+    if (int rc = check_shape(d->m, d->n, d->k)) return rc;
+    if (!valid_as(d->addr_space)) return fail(MIW_ERR_INVALID_AS, "Invalid address space for WMMA: %d", d->addr_space);
+    if (!valid_layout(d->a_layout) || !valid_layout(d->b_layout) || !valid_layout(d->c_layout) ||
+        !valid_layout(d->d_layout))
+        return fail(MIW_ERR_INVALID_LAYOUT, "Invalid layout for WMMA: a=%d b=%d c=%d d=%d", d->a_layout, d->b_layout,
+                    d->c_layout, d->d_layout);
+    if (!valid_dtype(d->c_type) || !valid_dtype(d->d_type))
+        return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: c=%d d=%d", d->c_type, d->d_type);
+    if (!A || !B || !D || (d->use_c && !C)) return fail(MIW_ERR_NULL_POINTER, "wmma_mac: null operand pointer");
+    const long lda = d->lda ? d->lda : 16, ldb = d->ldb ? d->ldb : 16, ldc = d->ldc ? d->ldc : 16,
+               ldd = d->ldd ? d->ldd : 16;
+    if (lda < 16 || ldb < 16 || ldc < 16 || ldd < 16)
+        return fail(MIW_ERR_INVALID_VALUE, "wmma_mac: leading dimension smaller than the tile");
+    if (((uintptr_t)A & 1) || ((uintptr_t)B & 1) || ((uintptr_t)D & (dtype_size(d->d_type) - 1)) ||
+        (d->use_c && ((uintptr_t)C & (dtype_size(d->c_type) - 1))))
+        return fail(MIW_ERR_MISALIGNED, "wmma_mac: operand pointer not aligned to its element type");
+    HIP_TRY(miw::launch_wmma_mac(d->c_type, d->d_type, A, B, C, D, lda, ldb, ldc, ldd, d->a_layout == MIW_ROW_MAJOR,
+                                 d->b_layout == MIW_ROW_MAJOR, d->c_layout == MIW_ROW_MAJOR,
+                                 d->d_layout == MIW_ROW_MAJOR, d->use_c != 0, d->addr_space == MIW_AS_SHARED, d->alpha,
+                                 d->beta, as_stream(stream)));
+    return 0;
+}
+
+// ------------------------------------------------------------------ GEMM ---
+
+int miw_gemm_variant_count(void) { return miw::tiled_variant_count() + 1; }
+
+int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out)
+{
+    if (!out) return fail(MIW_ERR_NULL_POINTER, "gemm_variant_info: null output");
+    const int nt = miw::tiled_variant_count();
+    if (variant < 1 || variant > nt + 1) return fail(MIW_ERR_INVALID_VALUE, "gemm_variant_info: unknown variant %d", variant);
+    memset(out, 0, sizeof(*out));
+    if (variant == nt + 1) {
+        snprintf(out->name, sizeof(out->name), "fragment_ops");
+        out->block_m = 16; out->block_n = 16; out->block_k = 16;
+        out->waves_m = 1; out->waves_n = 1; out->stages = 1; out->lds_bytes = 0; out->fragment_ops = 1;
+        return 0;
+    }
+    const miw::tiled_variant &v = miw::tiled_variant_at(variant - 1);
+    snprintf(out->name, sizeof(out->name), "%s", v.name);
+    out->block_m = v.bm; out->block_n = v.bn; out->block_k = v.bk;
+    out->waves_m = v.wm; out->waves_n = v.wn; out->stages = v.stages; out->lds_bytes = v.lds_bytes;
+    return 0;
+}
+
+int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant)
+{
+    if (!variant) return fail(MIW_ERR_NULL_POINTER, "gemm_pick_variant: null output");
+    miw::gemm_params p;
+    bool f16acc;
+    // Alignment of real pointers cannot be known here: assume aligned operands.
+    static char dummy alignas(16);
+    if (int rc = resolve_gemm(desc, &dummy, &dummy, &dummy, &dummy, &p, &f16acc)) return rc;
+    *variant = pick_variant(p, desc->c_type, desc->d_type, f16acc, desc->acc_chunk);
+    return 0;
+}
+
+int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk)
+{
+    if (!acc_chunk) return fail(MIW_ERR_NULL_POINTER, "gemm_acc_chunk: null output");
+    int v = 0;
+    if (int rc = miw_gemm_pick_variant(desc, &v)) return rc;
+    if (desc->variant != 0) v = desc->variant;
+    *acc_chunk = v == miw::tiled_variant_count() + 1 ? 16 : miw::tiled_f16acc_chunk();
+    return 0;
+}
+
+int miw_gemm(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream)
+{
+    miw::gemm_params p;
+    bool f16acc;
+    if (int rc = resolve_gemm(desc, A, B, C, D, &p, &f16acc)) return rc;
+    return run_gemm(desc, p, f16acc, as_stream(stream));
+}
+
+int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream,
+                   int warmup, int iters, float *ms_each)
+{
+    if (iters < 1 || warmup < 0 || !ms_each) return fail(MIW_ERR_INVALID_VALUE, "gemm_bench: bad warmup/iters/output");
+    miw::gemm_params p;
+    bool f16acc;
+    if (int rc = resolve_gemm(desc, A, B, C, D, &p, &f16acc)) return rc;
+    hipStream_t s = as_stream(stream);
+    for (int i = 0; i < warmup; i++)
+        if (int rc = run_gemm(desc, p, f16acc, s)) return rc;
+    std::vector<hipEvent_t> ev((size_t)iters + 1);
+    for (auto &e : ev) HIP_TRY(hipEventCreate(&e));
+    int rc = 0;
+    hipError_t he = hipEventRecord(ev[0], s);
+    for (int i = 0; i < iters && rc == 0 && he == hipSuccess; i++) {
+        rc = run_gemm(desc, p, f16acc, s);
+        if (rc == 0) he = hipEventRecord(ev[(size_t)i + 1], s);
+    }
+    if (rc == 0 && he == hipSuccess) he = hipEventSynchronize(ev[(size_t)iters]);
+    for (int i = 0; i < iters && rc == 0 && he == hipSuccess; i++)
+        he = hipEventElapsedTime(&ms_each[i], ev[(size_t)i], ev[(size_t)i + 1]);
+    for (auto &e : ev) (void)hipEventDestroy(e);
+    if (rc) return rc;
+    if (he != hipSuccess) return hip_fail(he, "gemm_bench");
+    return 0;
+}
+
+int miw_mfma_peak_probe(int iters, double *tflops, void *stream)
+{
+    if (!tflops || iters < 1) return fail(MIW_ERR_INVALID_VALUE, "mfma_peak_probe: bad arguments");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    const int blocks = prop.multiProcessorCount * 2;  // 8 wavefronts per CU
+    float *sink = nullptr;
+    HIP_TRY(hipMalloc((void **)&sink, 4));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipStream_t s = as_stream(stream);
+    hipError_t he = hipEventCreate(&e0);
+    if (he == hipSuccess) he = hipEventCreate(&e1);
+    if (he == hipSuccess) he = miw::launch_mfma_peak(blocks, 16, sink, s);  // warm-up
+    if (he == hipSuccess) he = hipEventRecord(e0, s);
+    if (he == hipSuccess) he = miw::launch_mfma_peak(blocks, iters, sink, s);
+    if (he == hipSuccess) he = hipEventRecord(e1, s);
+    if (he == hipSuccess) he = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    if (he != hipSuccess) return hip_fail(he, "mfma_peak_probe");
+    // per wavefront and iteration: 4 x 8 MFMAs of 16*16*32*2 flop
+    const double flop = (double)blocks * 4.0 * (double)iters * 32.0 * 16384.0;
+    *tflops = flop / ((double)ms * 1e-3) / 1e12;
+    return 0;
+}
+
+int miw_copy_probe(void *dst, const void *src, size_t bytes, void *stream)
+{
+    if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "copy_probe: null pointer");
+    if (((uintptr_t)dst | (uintptr_t)src | bytes) & 15) return fail(MIW_ERR_MISALIGNED, "copy_probe: needs 16-byte multiples");
+    HIP_TRY(miw::launch_copy(dst, src, bytes, as_stream(stream)));
+    return 0;
+}
+
+// -------------------------------------------------------- generic launch ---
+
+int miw_kernel_count(void) { return (int)registry().size(); }
+
+int miw_kernel_name(int index, char *buf, size_t buflen)
+{
+    if (!buf || buflen == 0) return fail(MIW_ERR_NULL_POINTER, "kernel_name: null buffer");
+    if (index < 0 || index >= (int)registry().size()) return fail(MIW_ERR_INVALID_VALUE, "kernel_name: index %d out of range", index);
+    snprintf(buf, buflen, "%s", registry()[(size_t)index].name.c_str());
+    return 0;
+}
+
+int miw_kernel_lookup(const char *name, void **kernel)
+{
+    if (!name || !kernel) return fail(MIW_ERR_NULL_POINTER, "kernel_lookup: null argument");
+    for (auto &k : registry())
+        if (k.name == name) {
+            *kernel = (void *)k.fn;
+            return 0;
+        }
+    *kernel = nullptr;
+    return fail(MIW_ERR_NOT_FOUND, "kernel_lookup: no kernel named '%s'", name);
+}
+
+int miw_kernel_attributes_get(void *kernel, miw_kernel_attributes *out)
+{
+    if (!kernel || !out) return fail(MIW_ERR_NULL_POINTER, "kernel_attributes: null argument");
+    hipFuncAttributes a;
+    HIP_TRY(hipFuncGetAttributes(&a, kernel));
+    out->num_regs = a.numRegs;
+    out->max_threads_per_block = a.maxThreadsPerBlock;
+    out->static_shared_bytes = a.sharedSizeBytes;
+    out->local_bytes = a.localSizeBytes;
+    out->const_bytes = a.constSizeBytes;
+    return 0;
+}
+
+int miw_kernel_occupancy(void *kernel, size_t dynamic_shmem, int *min_grid, int *block)
+{
+    if (!kernel || !min_grid || !block) return fail(MIW_ERR_NULL_POINTER, "kernel_occupancy: null argument");
+    HIP_TRY(hipOccupancyMaxPotentialBlockSize(min_grid, block, kernel, dynamic_shmem, 0));
+    return 0;
+}
+
+int miw_launch(void *kernel, const unsigned grid[3], const unsigned block[3], unsigned shmem, void *stream, void **args)
+{
+    if (!kernel || !grid || !block) return fail(MIW_ERR_NULL_POINTER, "launch: null argument");
+    bool known = false;
+    for (auto &k : registry()) known = known || (void *)k.fn == kernel;
+    if (!known) return fail(MIW_ERR_NOT_FOUND, "launch: not a kernel of this library");
+    const unsigned long threads = (unsigned long)block[0] * block[1] * block[2];
+    if (threads == 0 || (unsigned long)grid[0] * grid[1] * grid[2] == 0)
+        return fail(MIW_ERR_INVALID_VALUE, "launch: empty grid or block");
+    hipFuncAttributes a;
+    HIP_TRY(hipFuncGetAttributes(&a, kernel));
+    if (threads > (unsigned long)a.maxThreadsPerBlock)
+        return fail((int)hipErrorInvalidConfiguration, "launch: %lu threads per block exceed the kernel's maximum %d", threads,
+                    a.maxThreadsPerBlock);
+    HIP_TRY(hipLaunchKernel(kernel, dim3(grid[0], grid[1], grid[2]), dim3(block[0], block[1], block[2]), args, shmem,
+                            as_stream(stream)));
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,420 @@
+// One-wavefront kernels behind the op-granular fragment entry points, the fused
+// multiply-accumulate of examples/wmma/high-level.jl, and the GEMM written
+// directly with the fragment API (one wavefront per 16x16 output tile, the
+// "D of one mma is C of the next" chain of docs/src/device/wmma.md:51-52).
+#include "kernels.hpp"
+#include "wmma_fragment.hpp"
+
+namespace miw {
+
+using cfg_f32 = config<16, 16, 16, float>;
+using cfg_f16 = config<16, 16, 16, half_t>;
+
+// ------------------------------------------------------------ helpers ------
+
+// Copy a 16x16 tile (leading dimension `stride`, layout l) into an LDS tile of
+// leading dimension 16 with the same layout, as the reference's shared-memory
+// tests fill @cuStaticSharedMem(T, 256) (test/device/wmma.jl:42-46).
+template <class T>
+__device__ inline void stage_tile_to_lds(T *lds, const T *addr, long stride, layout l)
+{
+    for (int e = lane_id(); e < 256; e += 64) {
+        int i = e & 15, j = e >> 4;
+        lds[tile_offset(l, i, j, 16)] = addr[tile_offset(l, i, j, stride)];
+    }
+    __syncthreads();
+}
+
+template <class T>
+__device__ inline void unstage_tile_from_lds(T *addr, const T *lds, long stride, layout l)
+{
+    __syncthreads();
+    for (int e = lane_id(); e < 256; e += 64) {
+        int i = e & 15, j = e >> 4;
+        addr[tile_offset(l, i, j, stride)] = lds[tile_offset(l, i, j, 16)];
+    }
+}
+
+template <layout L, class PtrT>
+__device__ inline void load_ab_to_image(int use, PtrT p, long stride, half_t *img)
+{
+    const int ln = lane_id();
+    if (use == 0) {
+        auto f = load_a<cfg_f32, L>(p, stride);
+        for (int i = 0; i < 4; i++) img[ln * 4 + i] = f.x[i];
+    } else {
+        auto f = load_b<cfg_f32, L>(p, stride);
+        for (int i = 0; i < 4; i++) img[ln * 4 + i] = f.x[i];
+    }
+}
+
+// --------------------------------------------------------- load kernels ----
+
+// use: 0 = a, 1 = b, 2 = c.  as_mode: 0 generic, 1 global, 3 shared.
+template <class T>
+__global__ __launch_bounds__(64) void k_frag_load(int use, int row_major, int as_mode, const T *addr, long stride, T *img)
+{
+    __shared__ __attribute__((aligned(32))) T lds[256];
+    const layout l = row_major ? layout::row_major : layout::col_major;
+    const int ln = lane_id();
+    if (as_mode == 3) {
+        stage_tile_to_lds(lds, addr, stride, l);
+        const MIW_LDS T *p = (const MIW_LDS T *)lds;
+        if (use == 2) {
+            auto f = load_c<cfg_f32, T>(p, 16, l);
+            for (int i = 0; i < 4; i++) img[ln * 4 + i] = f.x[i];
+        } else if constexpr (__is_same(T, half_t)) {
+            if (row_major) load_ab_to_image<layout::row_major>(use, p, 16, img);
+            else load_ab_to_image<layout::col_major>(use, p, 16, img);
+        }
+    } else {
+        if (use == 2) {
+            auto f = load_c<cfg_f32, T>(addr, stride, l);
+            for (int i = 0; i < 4; i++) img[ln * 4 + i] = f.x[i];
+        } else if constexpr (__is_same(T, half_t)) {
+            if (row_major) load_ab_to_image<layout::row_major>(use, addr, stride, img);
+            else load_ab_to_image<layout::col_major>(use, addr, stride, img);
+        }
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(64) void k_frag_store(int row_major, int as_mode, T *addr, const T *img, long stride)
+{
+    __shared__ __attribute__((aligned(32))) T lds[256];
+    using cfg = config<16, 16, 16, T>;
+    const layout l = row_major ? layout::row_major : layout::col_major;
+    const int ln = lane_id();
+    fragment<accumulator, 16, 16, 16, T, layout::unspecified> d;
+    for (int i = 0; i < 4; i++) d.x[i] = img[ln * 4 + i];
+    if (as_mode == 3) {
+        store_d<cfg, T>((MIW_LDS T *)lds, d, 16, l);
+        unstage_tile_from_lds(addr, lds, stride, l);
+    } else {
+        store_d<cfg, T>(addr, d, stride, l);
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(64) void k_frag_fill(T value, T *img)
+{
+    auto f = fill_c<cfg_f32, T>(value);
+    const int ln = lane_id();
+    for (int i = 0; i < 4; i++) img[ln * 4 + i] = f.x[i];
+}
+
+// out[i] = s op in[i], computed in T as Julia's broadcast over a tuple of T does.
+template <class T>
+__global__ void k_frag_map(int op, T s, const T *in, T *out, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = op == 0 ? (T)(s * in[i]) : (T)(s + in[i]);
+}
+
+template <class CT, class DT>
+__global__ __launch_bounds__(64) void k_frag_mma(const half_t *a_img, const half_t *b_img, const CT *c_img, DT *d_img)
+{
+    using cfg = config<16, 16, 16, DT>;
+    const int ln = lane_id();
+    fragment<matrix_a, 16, 16, 16, half_t, layout::col_major> a;
+    fragment<matrix_b, 16, 16, 16, half_t, layout::col_major> b;
+    fragment<accumulator, 16, 16, 16, CT, layout::unspecified> c;
+    for (int i = 0; i < 4; i++) {
+        a.x[i] = a_img[ln * 4 + i];
+        b.x[i] = b_img[ln * 4 + i];
+        c.x[i] = c_img[ln * 4 + i];
+    }
+    auto d = mma<cfg>(a, b, c);
+    for (int i = 0; i < 4; i++) d_img[ln * 4 + i] = d.x[i];
+}
+
+// ------------------------------------------------- fused single-tile MAC ---
+
+struct mac_args {
+    const half_t *A;
+    const half_t *B;
+    const void *C;
+    void *D;
+    long lda, ldb, ldc, ldd;
+    int a_row, b_row, c_row, d_row;
+    int use_c;
+    int shared;
+    float alpha, beta;
+};
+
+template <class CT, class DT>
+__global__ __launch_bounds__(64) void k_wmma_mac(mac_args p)
+{
+    using cfg = config<16, 16, 16, DT>;
+    __shared__ __attribute__((aligned(32))) half_t lds_a[256];
+    __shared__ __attribute__((aligned(32))) half_t lds_b[256];
+    __shared__ __attribute__((aligned(32))) CT lds_c[256];
+    __shared__ __attribute__((aligned(32))) DT lds_d[256];
+
+    const layout lc = p.c_row ? layout::row_major : layout::col_major;
+    const layout ld = p.d_row ? layout::row_major : layout::col_major;
+
+    fragment<matrix_a, 16, 16, 16, half_t, layout::col_major> a;
+    fragment<matrix_b, 16, 16, 16, half_t, layout::col_major> b;
+    fragment<accumulator, 16, 16, 16, CT, layout::unspecified> c;
+
+    if (p.shared) {
+        stage_tile_to_lds(lds_a, p.A, p.lda, p.a_row ? layout::row_major : layout::col_major);
+        stage_tile_to_lds(lds_b, p.B, p.ldb, p.b_row ? layout::row_major : layout::col_major);
+        const MIW_LDS half_t *pa = (const MIW_LDS half_t *)lds_a;
+        const MIW_LDS half_t *pb = (const MIW_LDS half_t *)lds_b;
+        auto ar = load_a<cfg, layout::row_major>(pa, 16);
+        auto ac = load_a<cfg, layout::col_major>(pa, 16);
+        auto br = load_b<cfg, layout::row_major>(pb, 16);
+        auto bc = load_b<cfg, layout::col_major>(pb, 16);
+        for (int i = 0; i < 4; i++) {
+            a.x[i] = p.a_row ? ar.x[i] : ac.x[i];
+            b.x[i] = p.b_row ? br.x[i] : bc.x[i];
+        }
+        if (p.use_c) {
+            stage_tile_to_lds(lds_c, (const CT *)p.C, p.ldc, lc);
+            c = load_c<cfg, CT>((const MIW_LDS CT *)lds_c, 16, lc);
+        }
+    } else {
+        if (p.a_row) {
+            auto t = load_a<cfg, layout::row_major>(p.A, p.lda);
+            for (int i = 0; i < 4; i++) a.x[i] = t.x[i];
+        } else {
+            a = load_a<cfg, layout::col_major>(p.A, p.lda);
+        }
+        if (p.b_row) {
+            auto t = load_b<cfg, layout::row_major>(p.B, p.ldb);
+            for (int i = 0; i < 4; i++) b.x[i] = t.x[i];
+        } else {
+            b = load_b<cfg, layout::col_major>(p.B, p.ldb);
+        }
+        if (p.use_c) c = load_c<cfg, CT>((const CT *)p.C, p.ldc, lc);
+    }
+    if (!p.use_c) c = fill_c<cfg, CT>((CT)0);
+
+    // a_frag = alpha .* a_frag ; c_frag = beta .* c_frag  (test/device/wmma.jl:223-224)
+    a = scale((half_t)p.alpha, a);
+    c = scale((CT)p.beta, c);
+
+    auto d = mma<cfg>(a, b, c);
+
+    if (p.shared) {
+        store_d<cfg, DT>((MIW_LDS DT *)lds_d, d, 16, ld);
+        unstage_tile_from_lds((DT *)p.D, lds_d, p.ldd, ld);
+    } else {
+        store_d<cfg, DT>((DT *)p.D, d, p.ldd, ld);
+    }
+}
+
+// ------------------------------------------------ GEMM from fragment ops ---
+
+// One wavefront per 16x16 tile of D, four wavefronts per workgroup.
+// fp32 accumulate: acc = 0; acc = mma(a, b, acc) over K; D = alpha*acc + beta*C.
+// fp16 accumulate: acc = half(beta*C); acc = half(acc + alpha * (a*b)) per 16 k.
+template <class CT, class DT, bool F16ACC>
+__global__ __launch_bounds__(256) void k_gemm_fragops(gemm_params p)
+{
+    using cfg32 = config<16, 16, 16, float>;
+    const int wave = threadIdx.x >> 6;
+    const long tiles_m = p.M / 16, tiles_n = p.N / 16;
+    const long tile = (long)blockIdx.x * 4 + wave;
+    if (tile >= tiles_m * tiles_n) return;
+    const long tm = tile % tiles_m, tn = tile / tiles_m;
+    const long bt = blockIdx.y;
+
+    const half_t *A = p.A + bt * p.sa;
+    const half_t *B = p.B + bt * p.sb;
+    const CT *C = (const CT *)p.C + bt * p.sc;
+    DT *D = (DT *)p.D + bt * p.sd;
+
+    const layout la = p.a_row ? layout::row_major : layout::col_major;
+    const layout lb = p.b_row ? layout::row_major : layout::col_major;
+    const layout lc = p.c_row ? layout::row_major : layout::col_major;
+    const layout ld = p.d_row ? layout::row_major : layout::col_major;
+
+    const CT *Ct = C + tile_offset(lc, (int)(tm * 16), 0, p.ldc) + tile_offset(lc, 0, (int)(tn * 16), p.ldc);
+    DT *Dt = D + tile_offset(ld, (int)(tm * 16), 0, p.ldd) + tile_offset(ld, 0, (int)(tn * 16), p.ldd);
+
+    fragment<accumulator, 16, 16, 16, float, layout::unspecified> cin = fill_c<cfg32, float>(0.f);
+    if (p.use_c) {
+        auto cf = load_c<cfg32, CT>(Ct, p.ldc, lc);
+        for (int i = 0; i < 4; i++) cin.x[i] = (float)cf.x[i];
+    }
+
+    fragment<accumulator, 16, 16, 16, float, layout::unspecified> acc;
+    if constexpr (F16ACC) {
+        for (int i = 0; i < 4; i++) acc.x[i] = (float)(half_t)(p.beta * cin.x[i]);
+    } else {
+        acc = fill_c<cfg32, float>(0.f);
+    }
+
+    for (long k0 = 0; k0 < p.K; k0 += 16) {
+        const half_t *At = A + (la == layout::col_major ? tm * 16 + k0 * p.lda : tm * 16 * p.lda + k0);
+        const half_t *Bt = B + (lb == layout::col_major ? k0 + tn * 16 * p.ldb : k0 * p.ldb + tn * 16);
+        fragment<matrix_a, 16, 16, 16, half_t, layout::col_major> a;
+        fragment<matrix_b, 16, 16, 16, half_t, layout::col_major> b;
+        if (p.a_row) {
+            auto t = load_a<cfg32, layout::row_major>(At, p.lda);
+            for (int i = 0; i < 4; i++) a.x[i] = t.x[i];
+        } else {
+            a = load_a<cfg32, layout::col_major>(At, p.lda);
+        }
+        if (p.b_row) {
+            auto t = load_b<cfg32, layout::row_major>(Bt, p.ldb);
+            for (int i = 0; i < 4; i++) b.x[i] = t.x[i];
+        } else {
+            b = load_b<cfg32, layout::col_major>(Bt, p.ldb);
+        }
+        if constexpr (F16ACC) {
+            if (p.alpha == 1.0f) {
+                acc = mma<cfg32>(a, b, acc);
+            } else {
+                auto t = mma<cfg32>(a, b, fill_c<cfg32, float>(0.f));
+                for (int i = 0; i < 4; i++) acc.x[i] = __builtin_fmaf(p.alpha, t.x[i], acc.x[i]);
+            }
+            for (int i = 0; i < 4; i++) acc.x[i] = (float)(half_t)acc.x[i];
+        } else {
+            acc = mma<cfg32>(a, b, acc);
+        }
+    }
+
+    fragment<accumulator, 16, 16, 16, DT, layout::unspecified> d;
+    if constexpr (F16ACC) {
+        for (int i = 0; i < 4; i++) d.x[i] = (DT)acc.x[i];
+    } else {
+        for (int i = 0; i < 4; i++) {
+            float v = p.alpha * acc.x[i];
+            if (p.use_c) v = __builtin_fmaf(p.beta, cin.x[i], v);
+            d.x[i] = (DT)v;
+        }
+    }
+    store_d<config<16, 16, 16, DT>, DT>(Dt, d, p.ldd, ld);
+}
+
+// ------------------------------------------------------------ launchers ----
+
+hipError_t launch_frag_load(int use, int dtype, int row_major, int as_mode, const void *addr, long stride, void *img,
+                            hipStream_t s)
+{
+    if (dtype == 0)
+        hipLaunchKernelGGL(k_frag_load<half_t>, dim3(1), dim3(64), 0, s, use, row_major, as_mode, (const half_t *)addr,
+                           stride, (half_t *)img);
+    else
+        hipLaunchKernelGGL(k_frag_load<float>, dim3(1), dim3(64), 0, s, use, row_major, as_mode, (const float *)addr,
+                           stride, (float *)img);
+    return hipGetLastError();
+}
+
+hipError_t launch_frag_store(int dtype, int row_major, int as_mode, void *addr, const void *img, long stride,
+                             hipStream_t s)
+{
+    if (dtype == 0)
+        hipLaunchKernelGGL(k_frag_store<half_t>, dim3(1), dim3(64), 0, s, row_major, as_mode, (half_t *)addr,
+                           (const half_t *)img, stride);
+    else
+        hipLaunchKernelGGL(k_frag_store<float>, dim3(1), dim3(64), 0, s, row_major, as_mode, (float *)addr,
+                           (const float *)img, stride);
+    return hipGetLastError();
+}
+
+hipError_t launch_frag_fill(int dtype, float value, void *img, hipStream_t s)
+{
+    if (dtype == 0) hipLaunchKernelGGL(k_frag_fill<half_t>, dim3(1), dim3(64), 0, s, (half_t)value, (half_t *)img);
+    else hipLaunchKernelGGL(k_frag_fill<float>, dim3(1), dim3(64), 0, s, value, (float *)img);
+    return hipGetLastError();
+}
+
+hipError_t launch_frag_map(int dtype, int op, float scalar, const void *in, void *out, size_t n, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    dim3 grid((unsigned)((n + 255) / 256));
+    if (dtype == 0)
+        hipLaunchKernelGGL(k_frag_map<half_t>, grid, dim3(256), 0, s, op, (half_t)scalar, (const half_t *)in,
+                           (half_t *)out, n);
+    else
+        hipLaunchKernelGGL(k_frag_map<float>, grid, dim3(256), 0, s, op, scalar, (const float *)in, (float *)out, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_frag_mma(int c_type, int d_type, const void *a, const void *b, const void *c, void *d, hipStream_t s)
+{
+    const half_t *ha = (const half_t *)a, *hb = (const half_t *)b;
+    if (c_type == 0 && d_type == 0)
+        hipLaunchKernelGGL((k_frag_mma<half_t, half_t>), dim3(1), dim3(64), 0, s, ha, hb, (const half_t *)c, (half_t *)d);
+    else if (c_type == 0 && d_type == 1)
+        hipLaunchKernelGGL((k_frag_mma<half_t, float>), dim3(1), dim3(64), 0, s, ha, hb, (const half_t *)c, (float *)d);
+    else if (c_type == 1 && d_type == 0)
+        hipLaunchKernelGGL((k_frag_mma<float, half_t>), dim3(1), dim3(64), 0, s, ha, hb, (const float *)c, (half_t *)d);
+    else
+        hipLaunchKernelGGL((k_frag_mma<float, float>), dim3(1), dim3(64), 0, s, ha, hb, (const float *)c, (float *)d);
+    return hipGetLastError();
+}
+
+hipError_t launch_wmma_mac(int c_type, int d_type, const void *A, const void *B, const void *C, void *D, long lda,
+                           long ldb, long ldc, long ldd, int a_row, int b_row, int c_row, int d_row, int use_c,
+                           int shared, float alpha, float beta, hipStream_t s)
+{
+    mac_args p{(const half_t *)A, (const half_t *)B, C, D, lda, ldb, ldc, ldd, a_row, b_row, c_row, d_row,
+               use_c, shared, alpha, beta};
+    if (c_type == 0 && d_type == 0) hipLaunchKernelGGL((k_wmma_mac<half_t, half_t>), dim3(1), dim3(64), 0, s, p);
+    else if (c_type == 0 && d_type == 1) hipLaunchKernelGGL((k_wmma_mac<half_t, float>), dim3(1), dim3(64), 0, s, p);
+    else if (c_type == 1 && d_type == 0) hipLaunchKernelGGL((k_wmma_mac<float, half_t>), dim3(1), dim3(64), 0, s, p);
+    else hipLaunchKernelGGL((k_wmma_mac<float, float>), dim3(1), dim3(64), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_fragops(const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s)
+{
+    const long tiles = (p.M / 16) * (p.N / 16);
+    dim3 grid((unsigned)((tiles + 3) / 4), (unsigned)p.batch);
+    if (f16acc) {
+        hipLaunchKernelGGL((k_gemm_fragops<half_t, half_t, true>), grid, dim3(256), 0, s, p);
+    } else if (c_type == 0 && d_type == 0) {
+        hipLaunchKernelGGL((k_gemm_fragops<half_t, half_t, false>), grid, dim3(256), 0, s, p);
+    } else if (c_type == 0 && d_type == 1) {
+        hipLaunchKernelGGL((k_gemm_fragops<half_t, float, false>), grid, dim3(256), 0, s, p);
+    } else if (c_type == 1 && d_type == 0) {
+        hipLaunchKernelGGL((k_gemm_fragops<float, half_t, false>), grid, dim3(256), 0, s, p);
+    } else {
+        hipLaunchKernelGGL((k_gemm_fragops<float, float, false>), grid, dim3(256), 0, s, p);
+    }
+    return hipGetLastError();
+}
+
+// Host stubs exported to the named-kernel registry.
+const void *frag_kernel_symbol(const char *name)
+{
+    struct entry { const char *n; const void *f; };
+    static const entry table[] = {
+        {"frag_load_f16", (const void *)k_frag_load<half_t>},
+        {"frag_load_f32", (const void *)k_frag_load<float>},
+        {"frag_store_f16", (const void *)k_frag_store<half_t>},
+        {"frag_store_f32", (const void *)k_frag_store<float>},
+        {"frag_fill_f16", (const void *)k_frag_fill<half_t>},
+        {"frag_fill_f32", (const void *)k_frag_fill<float>},
+        {"frag_map_f16", (const void *)k_frag_map<half_t>},
+        {"frag_map_f32", (const void *)k_frag_map<float>},
+        {"frag_mma_f16_f16", (const void *)k_frag_mma<half_t, half_t>},
+        {"frag_mma_f16_f32", (const void *)k_frag_mma<half_t, float>},
+        {"frag_mma_f32_f16", (const void *)k_frag_mma<float, half_t>},
+        {"frag_mma_f32_f32", (const void *)k_frag_mma<float, float>},
+        {"wmma_mac_f32_f32", (const void *)k_wmma_mac<float, float>},
+        {"gemm_fragops_f32_f32", (const void *)k_gemm_fragops<float, float, false>},
+    };
+    for (const auto &e : table)
+        if (!__builtin_strcmp(e.n, name)) return e.f;
+    return nullptr;
+}
+
+int frag_kernel_count() { return 14; }
+
+const char *frag_kernel_name(int i)
+{
+    static const char *names[] = {"frag_load_f16",    "frag_load_f32",    "frag_store_f16",   "frag_store_f32",
+                                  "frag_fill_f16",    "frag_fill_f32",    "frag_map_f16",     "frag_map_f32",
+                                  "frag_mma_f16_f16", "frag_mma_f16_f32", "frag_mma_f32_f16", "frag_mma_f32_f32",
+                                  "wmma_mac_f32_f32", "gemm_fragops_f32_f32"};
+    return (i >= 0 && i < 14) ? names[i] : nullptr;
+}
+
+}  // namespace miw

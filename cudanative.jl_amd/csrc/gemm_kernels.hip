@@ -1,0 +1,484 @@
+// LDS-tiled mixed-precision GEMM for gfx950: D = alpha * A*B + beta * C with
+// Float16 A and B, fp32 accumulation in v_mfma_f32_16x16x32_f16 (optionally
+// rounded to Float16 after every K-tile: the fp16-accumulate variant).
+//
+// It is the chain "D of one mma is C of the next" (CUDAnative.jl
+// docs/src/device/wmma.md:51-52) carried over K, with the fragment loads of
+// src/device/cuda/wmma.jl:507-530 split in two: global -> LDS by 16-byte
+// direct-to-LDS loads, LDS -> registers in the matrix cores' operand layout.
+//
+// Canonical problem.  The kernel computes P = X * Y where P is I x J and is
+// stored with I contiguous.  For a column-major D this is X = A, Y = B,
+// I = M, J = N; for a row-major D the host passes X = B^T, Y = A^T, I = N,
+// J = M (same memory, roles swapped), so both D layouts write 16 contiguous
+// bytes per lane.  X is "K-major" when its k index is contiguous in memory
+// (A row-major / B column-major) and "I-major" otherwise; likewise Y.
+//
+// LDS tile layouts (K-tile = 64 k-values, 16-byte chunks):
+//   K-major operand, R rows : chunk (r, c) of row r (8 chunks of 8 k-values)
+//       sits at chunk index r*8 + (c ^ ((r >> 1) & 7)).  A lane reads its 8
+//       k-values for the MFMA with one ds_read_b128; the XOR spreads the 16
+//       rows of a fragment over all banks.
+//   I-major operand (k rows of R contiguous i) : stored as 128-byte blocks of
+//       4 k-values x 16 i, one block = what 16 lanes fetch with one
+//       ds_read_b64_tr_b16 (the LDS transpose read), which hands each lane
+//       4 consecutive k-values of its row.  Block (k4, i16) with
+//       k4 = 4a + 2mid + lo sits at block index ((2a + lo)*(R/16) + i16)*2 + mid,
+//       so the four 16-lane groups of one read hit alternating 128-byte halves.
+//   Direct-to-LDS loads write lane-contiguous 1 KiB per wavefront instruction;
+//   the layouts above are produced by choosing which global chunk each lane
+//   fetches.
+#include "kernels.hpp"
+
+#include <utility>
+
+namespace miw {
+
+typedef _Float16 half_t;
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __fp16 fp16x4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+
+#define MIW_LDS __attribute__((address_space(3)))
+#define MIW_GLOBAL __attribute__((address_space(1)))
+
+constexpr int BK = 64;  // k-values per K-tile
+
+struct tiled_params {
+    const half_t *X;
+    const half_t *Y;
+    const void *C;
+    void *D;
+    int I, J, K;
+    long ldx, ldy, ldc, ldd;
+    long sx, sy, sc, sd;
+    int c_trans;  // C is stored with J contiguous (its layout differs from D's)
+    int use_c;
+    float alpha, beta;
+    int tiles_i, tiles_j, group_i;
+};
+
+// vmcnt(n) with expcnt/lgkmcnt left alone (gfx9 encoding).
+#define MIW_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+
+// One 16-byte-per-lane direct-to-LDS load: lane l fetches base + voff[l] and
+// the wavefront's 1 KiB lands at LDS byte lds_addr + 16*l.  Written as inline
+// assembly so that the compiler's wait-count pass does not serialise it with
+// the LDS reads of the other stage; completion is awaited explicitly with
+// MIW_WAIT_VMCNT before the barrier that publishes the tile.
+__device__ inline void lds_dma16(const void *base, unsigned voff, unsigned lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(base)
+                 : "memory", "m0");
+}
+
+// ------------------------------------------------------------ tile loader --
+template <int R, bool KMAJOR, int NT>
+struct tile_loader {
+    static constexpr int CHUNKS = R * 8;
+    static constexpr int NLOAD = CHUNKS / NT;
+    static_assert(CHUNKS % NT == 0, "tile must divide over the workgroup");
+
+    // Element offset, relative to the tile origin at k-tile 0, of the global
+    // chunk that lands in LDS chunk q.
+    __device__ static inline int source_offset(int q, int ld)
+    {
+        if constexpr (KMAJOR) {
+            const int r = q >> 3, cpos = q & 7;
+            const int c = cpos ^ ((r >> 1) & 7);
+            return r * ld + c * 8;
+        } else {
+            constexpr int R16 = R / 16;
+            const int b = q >> 3, kq = (q & 7) >> 1, hf = q & 1;
+            const int mid = b & 1, rest = b >> 1;
+            const int i16 = rest % R16, x = rest / R16;
+            const int k4 = 4 * (x >> 1) + 2 * mid + (x & 1);
+            return (4 * k4 + kq) * ld + 16 * i16 + 8 * hf;
+        }
+    }
+
+    // Byte offsets of this thread's chunks.
+    __device__ static inline void offsets(int tid, int ld, unsigned (&off)[NLOAD])
+    {
+#pragma unroll
+        for (int i = 0; i < NLOAD; i++) off[i] = 2u * (unsigned)source_offset(i * NT + tid, ld);
+    }
+
+    // base: uniform global address of the tile origin; lds_wave: this
+    // wavefront's first destination byte for load 0 (uniform).
+    __device__ static inline void issue(const half_t *base, const unsigned (&off)[NLOAD], unsigned lds_wave)
+    {
+#pragma unroll
+        for (int i = 0; i < NLOAD; i++) lds_dma16(base, off[i], lds_wave + (unsigned)(i * NT * 16));
+    }
+};
+
+// --------------------------------------------------------- fragment reads --
+// Lane byte offset (within the operand's LDS tile) of the fragment of MFMA
+// tile 0, k-step 0; tile t / k-step ks / half h add compile-time constants.
+template <int R, bool KMAJOR>
+struct frag_reader {
+    static constexpr int R16 = R / 16;
+    int base0, base1;  // K-major: one lane offset per k-step (the XOR involves ks)
+
+    __device__ inline void init(int wave_row0, int lane)
+    {
+        const int j = lane & 15, q = lane >> 4;
+        if constexpr (KMAJOR) {
+            const int r = wave_row0 + j;
+            base0 = (r * 8 + ((0 + q) ^ ((j >> 1) & 7))) * 16;
+            base1 = (r * 8 + ((4 + q) ^ ((j >> 1) & 7))) * 16;
+        } else {
+            base0 = ((2 * (q >> 1)) * R16 + wave_row0 / 16) * 256 + (q & 1) * 128 + j * 8;
+            base1 = 0;
+        }
+    }
+
+    template <int T, int KS>
+    __device__ inline half8_t read(MIW_LDS const char *tile) const
+    {
+        if constexpr (KMAJOR) {
+            const int off = (KS == 0 ? base0 : base1) + T * 2048;
+            return *(MIW_LDS const half8_t *)(tile + off);
+        } else {
+            const int off = base0 + KS * (4 * R16 * 256) + T * 256;
+            fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(tile + off));
+            fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(tile + off + R16 * 256));
+            uint2_t l2 = __builtin_bit_cast(uint2_t, lo), h2 = __builtin_bit_cast(uint2_t, hi);
+            uint4_t v = {l2[0], l2[1], h2[0], h2[1]};
+            return __builtin_bit_cast(half8_t, v);
+        }
+    }
+};
+
+__device__ inline float round_through_half(float v) { return (float)(half_t)v; }
+
+// ----------------------------------------------------------------- kernel --
+template <int BI, int BJ, int WI, int WJ, bool XK, bool YK, class CT, class DT, bool F16ACC>
+__global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
+{
+    constexpr int NT = WI * WJ * 64;
+    constexpr int WTI = BI / WI, WTJ = BJ / WJ;
+    constexpr int TI = WTI / 16, TJ = WTJ / 16;
+    constexpr int XBYTES = BI * BK * 2, YBYTES = BJ * BK * 2, STAGE = XBYTES + YBYTES;
+    using xload = tile_loader<BI, XK, NT>;
+    using yload = tile_loader<BJ, YK, NT>;
+
+    extern __shared__ __attribute__((aligned(128))) char smem[];
+    MIW_LDS char *lds = (MIW_LDS char *)smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wi = wave % WI, wj = wave / WI;
+
+    // Workgroup -> tile.  Consecutive workgroup ids go round-robin over the 8
+    // XCDs; give each XCD a contiguous run of tile ids so that workgroups that
+    // share X row-panels and Y column-panels share one L2, then walk the tile
+    // grid in groups of group_i tile-rows.
+    int tile_id;
+    {
+        const int total = p.tiles_i * p.tiles_j;
+        const int pid = blockIdx.x;
+        const int per = total >> 3, rem = total & 7;
+        const int xcd = pid & 7, loc = pid >> 3;
+        tile_id = xcd < rem ? xcd * (per + 1) + loc : rem * (per + 1) + (xcd - rem) * per + loc;
+    }
+    int ti0, tj0;
+    {
+        const int gsz = p.group_i * p.tiles_j;
+        const int gid = tile_id / gsz;
+        const int first = gid * p.group_i;
+        const int gi = min(p.tiles_i - first, p.group_i);
+        const int in = tile_id - gid * gsz;
+        ti0 = first + in % gi;
+        tj0 = in / gi;
+    }
+    const long bt = blockIdx.y;
+    const int i0 = ti0 * BI, j0 = tj0 * BJ;
+
+    const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
+    const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);
+    const long xstep = XK ? BK : (long)BK * p.ldx;
+    const long ystep = YK ? BK : (long)BK * p.ldy;
+
+    unsigned xoff[xload::NLOAD], yoff[yload::NLOAD];
+    xload::offsets(tid, (int)p.ldx, xoff);
+    yload::offsets(tid, (int)p.ldy, yoff);
+
+    frag_reader<BI, XK> xr;
+    frag_reader<BJ, YK> yr;
+    xr.init(wi * WTI, lane);
+    yr.init(wj * WTJ, lane);
+
+    const int q = lane >> 4, r = lane & 15;
+    const int row = i0 + wi * WTI + 4 * q;  // + 16*ti
+    const int col = j0 + wj * WTJ + r;      // + 16*tj
+    const CT *C = (const CT *)p.C + bt * p.sc;
+    DT *D = (DT *)p.D + bt * p.sd;
+
+    float4_t acc[TI][TJ];
+#pragma unroll
+    for (int a = 0; a < TI; a++)
+#pragma unroll
+        for (int b = 0; b < TJ; b++) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // C in the accumulator layout: 4 consecutive i of one column j per lane.
+    // `trans` (C stored with j contiguous) is uniform over the grid.
+    auto read_c = [&](int a, int b, bool trans) -> float4_t {
+        float4_t c;
+        const int ii = row + 16 * a, jj = col + 16 * b;
+        if (trans) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) c[v] = (float)C[(long)(ii + v) * p.ldc + jj];
+        } else if constexpr (__is_same(CT, float)) {
+            c = *(const float4_t *)(C + (long)jj * p.ldc + ii);
+        } else {
+            half4_t h = *(const half4_t *)(C + (long)jj * p.ldc + ii);
+            c = float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+        }
+        return c;
+    };
+
+    // First K-tile on its way before anything else.
+    const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
+    xload::issue(X, xoff, wave_dst);
+    yload::issue(Y, yoff, wave_dst + XBYTES);
+
+    if constexpr (F16ACC) {
+        // acc = half(beta * C): the Float16 accumulator starts as the C operand.
+        if (p.use_c) {
+            auto init = [&](bool trans) {
+#pragma unroll
+                for (int a = 0; a < TI; a++)
+#pragma unroll
+                    for (int b = 0; b < TJ; b++) {
+                        float4_t c = read_c(a, b, trans);
+#pragma unroll
+                        for (int v = 0; v < 4; v++) acc[a][b][v] = round_through_half(p.beta * c[v]);
+                    }
+            };
+            if (p.c_trans) init(true);
+            else init(false);
+        }
+    }
+
+    const int KT = p.K / BK;
+    for (int kt = 0; kt < KT; kt++) {
+        MIW_WAIT_VMCNT(0);
+        __syncthreads();
+        const int cur = (kt & 1) * STAGE;
+        if (kt + 1 < KT) {
+            X += xstep;
+            Y += ystep;
+            const int nxt = STAGE - cur;
+            xload::issue(X, xoff, wave_dst + nxt);
+            yload::issue(Y, yoff, wave_dst + nxt + XBYTES);
+        }
+        MIW_LDS const char *xt = lds + cur;
+        MIW_LDS const char *yt = lds + cur + XBYTES;
+
+        half8_t xf[2][TI], yf[2][TJ];
+        [&]<int... A>(__attribute__((unused)) std::integer_sequence<int, A...>) {
+            ((xf[0][A] = xr.template read<A, 0>(xt)), ...);
+            ((xf[1][A] = xr.template read<A, 1>(xt)), ...);
+        }(std::make_integer_sequence<int, TI>{});
+        [&]<int... B>(__attribute__((unused)) std::integer_sequence<int, B...>) {
+            ((yf[0][B] = yr.template read<B, 0>(yt)), ...);
+            ((yf[1][B] = yr.template read<B, 1>(yt)), ...);
+        }(std::make_integer_sequence<int, TJ>{});
+
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int a = 0; a < TI; a++)
+#pragma unroll
+                for (int b = 0; b < TJ; b++)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[ks][a], yf[ks][b], acc[a][b], 0, 0, 0);
+
+        if constexpr (F16ACC) {
+#pragma unroll
+            for (int a = 0; a < TI; a++)
+#pragma unroll
+                for (int b = 0; b < TJ; b++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) acc[a][b][v] = round_through_half(acc[a][b][v]);
+        }
+    }
+
+    // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
+    auto epilogue = [&](bool with_c, bool trans) {
+#pragma unroll
+        for (int b = 0; b < TJ; b++)
+#pragma unroll
+            for (int a = 0; a < TI; a++) {
+                float4_t v = acc[a][b];
+                if constexpr (!F16ACC) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] *= p.alpha;
+                    if (with_c) {
+                        float4_t c = read_c(a, b, trans);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
+                    }
+                }
+                DT *dst = D + (long)(col + 16 * b) * p.ldd + (row + 16 * a);
+                if constexpr (__is_same(DT, float)) {
+                    *(float4_t *)dst = v;
+                } else {
+                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    *(half4_t *)dst = h;
+                }
+            }
+    };
+    if (F16ACC || !p.use_c) epilogue(false, false);
+    else if (p.c_trans) epilogue(true, true);
+    else epilogue(true, false);
+}
+
+// --------------------------------------------------------------- variants --
+
+static const tiled_variant g_variants[] = {
+    // name                 bm   bn  bk  wm wn st  lds
+    {"tile256x256_w2x4", 256, 256, 64, 2, 4, 2, 2 * (256 + 256) * 128},
+    {"tile256x256_w4x2", 256, 256, 64, 4, 2, 2, 2 * (256 + 256) * 128},
+    {"tile256x128_w2x2", 256, 128, 64, 2, 2, 2, 2 * (256 + 128) * 128},
+    {"tile128x256_w2x2", 128, 256, 64, 2, 2, 2, 2 * (128 + 256) * 128},
+    {"tile128x128_w2x2", 128, 128, 64, 2, 2, 2, 2 * (128 + 128) * 128},
+    {"tile64x64_w2x2", 64, 64, 64, 2, 2, 2, 2 * (64 + 64) * 128},
+};
+
+int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }
+const tiled_variant &tiled_variant_at(int i) { return g_variants[i]; }
+int tiled_f16acc_chunk() { return BK; }
+
+template <int BI, int BJ, int WI, int WJ, class CT, class DT, bool F16ACC>
+static const void *pick_layout(bool xk, bool yk)
+{
+    if (xk && yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, true, true, CT, DT, F16ACC>;
+    if (xk && !yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, true, false, CT, DT, F16ACC>;
+    if (!xk && yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, false, true, CT, DT, F16ACC>;
+    return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, false, false, CT, DT, F16ACC>;
+}
+
+template <int BI, int BJ, int WI, int WJ>
+static const void *pick_types(bool xk, bool yk, int c_type, int d_type, bool f16acc)
+{
+    if (f16acc) return pick_layout<BI, BJ, WI, WJ, half_t, half_t, true>(xk, yk);
+    if (c_type == 0 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, half_t, half_t, false>(xk, yk);
+    if (c_type == 0 && d_type == 1) return pick_layout<BI, BJ, WI, WJ, half_t, float, false>(xk, yk);
+    if (c_type == 1 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, float, half_t, false>(xk, yk);
+    return pick_layout<BI, BJ, WI, WJ, float, float, false>(xk, yk);
+}
+
+// Tile shape in canonical (I, J) terms: bm applies to I, bn to J.
+static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, bool f16acc)
+{
+    switch (i) {
+        case 0: return pick_types<256, 256, 2, 4>(xk, yk, c_type, d_type, f16acc);
+        case 1: return pick_types<256, 256, 4, 2>(xk, yk, c_type, d_type, f16acc);
+        case 2: return pick_types<256, 128, 2, 2>(xk, yk, c_type, d_type, f16acc);
+        case 3: return pick_types<128, 256, 2, 2>(xk, yk, c_type, d_type, f16acc);
+        case 4: return pick_types<128, 128, 2, 2>(xk, yk, c_type, d_type, f16acc);
+        case 5: return pick_types<64, 64, 2, 2>(xk, yk, c_type, d_type, f16acc);
+    }
+    return nullptr;
+}
+
+const void *tiled_kernel_symbol(int i) { return pick_kernel(i, false, true, 1, 1, false); }
+
+hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type, bool f16acc, hipStream_t s)
+{
+    const tiled_variant &v = g_variants[i];
+    tiled_params p;
+    bool xk, yk;
+    if (!g.d_row) {
+        // P = D (M x N, M contiguous): X = A, Y = B
+        p.X = g.A; p.Y = g.B;
+        p.I = (int)g.M; p.J = (int)g.N;
+        p.ldx = g.lda; p.ldy = g.ldb; p.sx = g.sa; p.sy = g.sb;
+        xk = g.a_row != 0;   // A row-major: k contiguous
+        yk = g.b_row == 0;   // B column-major: k contiguous
+        p.c_trans = g.c_row != 0;
+    } else {
+        // P = D^T (N x M, N contiguous): X = B^T, Y = A^T
+        p.X = g.B; p.Y = g.A;
+        p.I = (int)g.N; p.J = (int)g.M;
+        p.ldx = g.ldb; p.ldy = g.lda; p.sx = g.sb; p.sy = g.sa;
+        xk = g.b_row == 0;
+        yk = g.a_row != 0;
+        p.c_trans = g.c_row == 0;
+    }
+    p.C = g.C; p.D = g.D;
+    p.K = (int)g.K;
+    p.ldc = g.ldc; p.ldd = g.ldd; p.sc = g.sc; p.sd = g.sd;
+    p.use_c = g.use_c;
+    p.alpha = g.alpha; p.beta = g.beta;
+    p.tiles_i = p.I / v.bm;
+    p.tiles_j = p.J / v.bn;
+    // Rows of tiles per raster group: about the square root of one XCD's share.
+    int per_xcd = (p.tiles_i * p.tiles_j + 7) / 8, gi = 1;
+    while ((gi * 2) * (gi * 2) <= per_xcd) gi *= 2;
+    p.group_i = gi < p.tiles_i ? gi : p.tiles_i;
+
+    const void *fn = pick_kernel(i, xk, yk, c_type, d_type, f16acc);
+    if (!fn) return hipErrorInvalidValue;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes);
+    if (e != hipSuccess) return e;
+    void *args[] = {&p};
+    dim3 grid((unsigned)(p.tiles_i * p.tiles_j), (unsigned)g.batch);
+    return hipLaunchKernel(fn, grid, dim3((unsigned)(v.wm * v.wn * 64)), args, (size_t)v.lds_bytes, s);
+}
+
+// ------------------------------------------------------------ probes -------
+
+// Register-resident MFMA chain: 8 independent accumulators per wavefront.
+__global__ __launch_bounds__(256) void k_mfma_peak(int iters, float *sink)
+{
+    half8_t a, b;
+    for (int i = 0; i < 8; i++) {
+        a[i] = (half_t)(0.001f * (float)(threadIdx.x + i));
+        b[i] = (half_t)(0.002f * (float)(threadIdx.x ^ i));
+    }
+    float4_t acc[8];
+    for (int i = 0; i < 8; i++) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[i], 0, 0, 0);
+    }
+    float s = 0.f;
+    for (int i = 0; i < 8; i++) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    if (s == 12345.678f) sink[0] = s;  // keeps the chain alive
+}
+
+hipError_t launch_mfma_peak(int blocks, int iters, float *sink, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_mfma_peak, dim3((unsigned)blocks), dim3(256), 0, s, iters, sink);
+    return hipGetLastError();
+}
+
+__global__ __launch_bounds__(256) void k_copy16(uint4_t *dst, const uint4_t *src, size_t n16)
+{
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+hipError_t launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s)
+{
+    size_t n16 = bytes / 16;
+    unsigned blocks = (unsigned)((n16 + 255) / 256);
+    if (blocks > 256u * 16u) blocks = 256u * 16u;
+    if (blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_copy16, dim3(blocks), dim3(256), 0, s, (uint4_t *)dst, (const uint4_t *)src, n16);
+    return hipGetLastError();
+}
+
+}  // namespace miw

@@ -1,0 +1,59 @@
+// Declarations shared by the kernel translation units and the C ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace miw {
+
+// Arguments of every GEMM kernel: D = alpha * A*B + beta * C, A (M x K) and
+// B (K x N) Float16, leading dimensions and batch strides in elements.
+struct gemm_params {
+    const _Float16 *A;
+    const _Float16 *B;
+    const void *C;
+    void *D;
+    long M, N, K;
+    long lda, ldb, ldc, ldd;
+    long sa, sb, sc, sd;
+    long batch;
+    int a_row, b_row, c_row, d_row;  // 1: row major, 0: column major
+    int use_c;
+    float alpha, beta;
+};
+
+// --- frag_kernels.hip
+hipError_t launch_frag_load(int use, int dtype, int row_major, int as_mode, const void *addr, long stride, void *img,
+                            hipStream_t s);
+hipError_t launch_frag_store(int dtype, int row_major, int as_mode, void *addr, const void *img, long stride,
+                             hipStream_t s);
+hipError_t launch_frag_fill(int dtype, float value, void *img, hipStream_t s);
+hipError_t launch_frag_map(int dtype, int op, float scalar, const void *in, void *out, size_t n, hipStream_t s);
+hipError_t launch_frag_mma(int c_type, int d_type, const void *a, const void *b, const void *c, void *d, hipStream_t s);
+hipError_t launch_wmma_mac(int c_type, int d_type, const void *A, const void *B, const void *C, void *D, long lda,
+                           long ldb, long ldc, long ldd, int a_row, int b_row, int c_row, int d_row, int use_c,
+                           int shared, float alpha, float beta, hipStream_t s);
+hipError_t launch_gemm_fragops(const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s);
+const void *frag_kernel_symbol(const char *name);
+int frag_kernel_count();
+const char *frag_kernel_name(int i);
+
+// --- gemm_kernels.hip
+struct tiled_variant {
+    const char *name;
+    int bm, bn, bk, wm, wn, stages, lds_bytes;
+};
+int tiled_variant_count();
+const tiled_variant &tiled_variant_at(int i);
+// acc_chunk the tiled fp16-accumulate kernels round at.
+int tiled_f16acc_chunk();
+// Launches tiled variant i.  The caller has checked divisibility by the tile,
+// 16-byte alignment of pointers and leading dimensions, and (for fp16
+// accumulate) alpha == 1 and c_type == d_type == Float16.
+hipError_t launch_gemm_tiled(int i, const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s);
+const void *tiled_kernel_symbol(int i);
+
+hipError_t launch_mfma_peak(int blocks, int iters, float *sink, hipStream_t s);
+hipError_t launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s);
+
+}  // namespace miw

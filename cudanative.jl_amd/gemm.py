@@ -1,0 +1,77 @@
+"""Tiled mixed-precision GEMM D = alpha*A*B + beta*C on the WMMA path.
+
+The reference ships no tiled GEMM; its contract is the chain of mma calls of
+docs/src/device/wmma.md:51-52 ("D of one multiply-accumulate is C of the next")
+over the whole K extent.  This module is the host call surface over miw_gemm.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from .array import DeviceArray
+from .wmma import ColMajor, RowMajor, get_hl_frag_info, get_hl_layout, Float16, Float32
+
+
+def _layout_code(L):
+    get_hl_layout(L)
+    return _lib.ROW_MAJOR if L is RowMajor else _lib.COL_MAJOR
+
+
+def _dtype_code(T):
+    return _lib.F16 if np.dtype(T) == np.float16 else _lib.F32
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    return x.ptr if isinstance(x, DeviceArray) else int(x)
+
+
+def make_desc(M, N, K, *, a_layout=ColMajor, b_layout=ColMajor, c_layout=ColMajor, d_layout=ColMajor,
+              c_type=Float32, d_type=Float32, acc_type=Float32, acc_chunk=0, alpha=1.0, beta=1.0, use_c=True,
+              batch=1, lda=0, ldb=0, ldc=0, ldd=0, stride_a=0, stride_b=0, stride_c=0, stride_d=0, variant=0):
+    get_hl_frag_info("c", c_type)
+    get_hl_frag_info("d", d_type)
+    get_hl_frag_info("c", acc_type)
+    return _lib.GemmDesc(M, N, K, lda, ldb, ldc, ldd, _layout_code(a_layout), _layout_code(b_layout),
+                         _layout_code(c_layout), _layout_code(d_layout), _dtype_code(c_type), _dtype_code(d_type),
+                         _dtype_code(acc_type), acc_chunk, float(alpha), float(beta), 1 if use_c else 0, batch,
+                         stride_a, stride_b, stride_c, stride_d, variant)
+
+
+def gemm(A, B, C, D, desc, stream=None):
+    """Launch D = alpha*A*B + beta*C (asynchronous).  A, B, C, D: DeviceArray or raw device address."""
+    _lib.check(_lib.load().miw_gemm(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), stream))
+
+
+def gemm_bench(A, B, C, D, desc, warmup=5, iters=20, stream=None):
+    """Per-launch durations in milliseconds, HIP events on the launch stream."""
+    ms = (ctypes.c_float * iters)()
+    _lib.check(_lib.load().miw_gemm_bench(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), stream,
+                                          warmup, iters, ms))
+    return np.array(ms[:], dtype=np.float64)
+
+
+def variants():
+    lib = _lib.load()
+    out = []
+    for v in range(1, lib.miw_gemm_variant_count() + 1):
+        info = _lib.GemmVariantInfo()
+        _lib.check(lib.miw_gemm_variant_info_get(v, ctypes.byref(info)))
+        out.append({"id": v, "name": info.name.decode(), "block": (info.block_m, info.block_n, info.block_k),
+                    "waves": (info.waves_m, info.waves_n), "stages": info.stages, "lds_bytes": info.lds_bytes,
+                    "fragment_ops": bool(info.fragment_ops)})
+    return out
+
+
+def pick_variant(desc):
+    v = ctypes.c_int()
+    _lib.check(_lib.load().miw_gemm_pick_variant(ctypes.byref(desc), ctypes.byref(v)))
+    return v.value
+
+
+def acc_chunk(desc):
+    v = ctypes.c_int()
+    _lib.check(_lib.load().miw_gemm_acc_chunk(ctypes.byref(desc), ctypes.byref(v)))
+    return v.value

@@ -1,0 +1,242 @@
+/*
+ * miwmma.h -- C ABI of libmiwmma.so: WMMA fragment operations and the tiled
+ * mixed-precision GEMM built on them, for AMD MI355X (gfx950, wave64, MFMA).
+ *
+ * This is the boundary that replaces, for the WMMA/GEMM path only, what
+ * CUDAnative.jl reaches through CUDAdrv and the NVPTX back end.  Each entry
+ * names the reference interface it stands in for (paths relative to the
+ * CUDAnative.jl v3.1.0 tree).
+ *
+ * Conventions
+ *   - every function returns 0 on success, a positive hipError_t when the HIP
+ *     runtime failed, or a negative MIW_ERR_* code when the library rejected the
+ *     arguments; miw_last_error() returns a thread-local message for the last
+ *     non-zero return on the calling thread.  Nothing throws or aborts.
+ *   - pointers named A, B, C, D, addr, frag are DEVICE pointers unless stated.
+ *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.
+ *     Launches are asynchronous; the caller keeps buffers alive until
+ *     miw_sync() (the GC.@preserve of src/execution.jl:105).
+ *   - the library retains no caller pointer past a call.
+ *   - a wavefront is 64 lanes: a fragment of the 16x16x16 tile holds 4 elements
+ *     per lane for every use (the reference's warp32 held 16/16/8,
+ *     src/device/cuda/wmma.jl:413-420).  A fragment image is the wavefront's
+ *     registers spilled to memory: element i of lane l at index l*4 + i.
+ */
+#ifndef MIWMMA_H
+#define MIWMMA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ enums -- */
+
+/* FragmentLayout: RowMajor / ColMajor (src/device/cuda/wmma.jl:313-338). */
+enum { MIW_ROW_MAJOR = 0, MIW_COL_MAJOR = 1 };
+/* Element types WMMA accepts (src/device/cuda/wmma.jl:11-15). */
+enum { MIW_F16 = 0, MIW_F32 = 1 };
+/* FragmentUse: MatrixA / MatrixB / Accumulator (src/device/cuda/wmma.jl:343-346). */
+enum { MIW_MATRIX_A = 0, MIW_MATRIX_B = 1, MIW_ACCUMULATOR = 2 };
+/* Address spaces, numbered as AS.Generic/Global/Shared (src/device/pointer.jl:11-27).
+   SHARED stages the tile through LDS inside the kernel and runs the LDS-pointer
+   overload of the fragment op, as test/device/wmma.jl:42-46,83-89 do. */
+enum { MIW_AS_GENERIC = 0, MIW_AS_GLOBAL = 1, MIW_AS_SHARED = 3 };
+/* Broadcast operators over a fragment (src/device/cuda/wmma.jl:703-716). */
+enum { MIW_OP_MUL = 0, MIW_OP_ADD = 1 };
+
+enum {
+    MIW_OK = 0,
+    MIW_ERR_INVALID_VALUE = -1,
+    MIW_ERR_INVALID_SHAPE = -2,   /* "Invalid shape for WMMA" (wmma.jl:450-453) */
+    MIW_ERR_INVALID_LAYOUT = -3,  /* "Invalid layout for WMMA" (wmma.jl:442-448) */
+    MIW_ERR_INVALID_TYPE = -4,    /* "Invalid element type for WMMA" (wmma.jl:460-477) */
+    MIW_ERR_INVALID_AS = -5,      /* "Invalid address space for WMMA" (wmma.jl:434-440) */
+    MIW_ERR_MISALIGNED = -6,
+    MIW_ERR_NULL_POINTER = -7,
+    MIW_ERR_NOT_INITIALIZED = -8,
+    MIW_ERR_UNSUPPORTED = -9,
+    MIW_ERR_NOT_FOUND = -10
+};
+
+/* -------------------------------------------------------------- lifecycle -- */
+
+/* Select the device and check it is a gfx950 part.  Replaces the lazy context
+   creation of src/init.jl:101-112 (context()) for one GPU. */
+int miw_init(int device);
+
+/* Message for the last failing call on this thread ("" if none). */
+const char *miw_last_error(void);
+
+typedef struct miw_device_info {
+    char name[128];
+    char arch[64];
+    int cu_count;
+    int wave_size;
+    int clock_mhz;          /* peak engine clock */
+    int mem_clock_mhz;
+    int mem_bus_bits;
+    int l2_bytes;
+    int max_threads_per_block;
+    size_t lds_per_block;   /* bytes a workgroup may allocate */
+    size_t hbm_bytes;
+    double peak_f16_tflops; /* cu_count * 4 SIMD * 1024 flop/clk * clock */
+} miw_device_info;
+
+/* Device properties (CUDAdrv device attributes used by src/execution.jl:418-426
+   warpsize helpers and by the occupancy callback). */
+int miw_device_info_get(miw_device_info *out);
+
+/* ----------------------------------------------------------------- memory -- */
+/* CuHostArray: Mem.alloc / Mem.free / unsafe_copyto! (src/array.jl:20-60). */
+int miw_malloc(void **out, size_t bytes);
+int miw_free(void *p);
+int miw_memcpy_h2d(void *dst, const void *src_host, size_t bytes);
+int miw_memcpy_d2h(void *dst_host, const void *src, size_t bytes);
+int miw_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int miw_memset(void *dst, int byte, size_t bytes);
+
+/* stream= keyword of @cuda (src/execution.jl:59-63); synchronize() */
+int miw_stream_create(void **out);
+int miw_stream_destroy(void *stream);
+int miw_sync(void *stream);
+
+/* CuEvent timing as used by test/perf/launch_overhead. */
+int miw_event_create(void **out);
+int miw_event_destroy(void *event);
+int miw_event_record(void *event, void *stream);
+int miw_event_synchronize(void *event);
+int miw_event_elapsed_ms(float *ms, void *start, void *stop);
+
+/* ------------------------------------------------------- fragment operations */
+/* Each call launches one wavefront (1 block x 64 threads; the reference
+   launches 1 x 32, examples/wmma/high-level.jl:46). */
+
+/* Elements per lane of a fragment: 4 for every (use, dtype) of the 16x16x16 tile. */
+int miw_frag_elems_per_lane(int use, int dtype);
+/* Bytes of a fragment image (64 lanes). */
+size_t miw_frag_image_bytes(int use, int dtype);
+
+/* load_a / load_b / load_c (src/device/cuda/wmma.jl:507-530;
+   llvm_wmma_load_* :104-137).  use selects a/b/c; A and B must be MIW_F16.
+   stride is the leading dimension in elements. M,N,K must be 16. */
+int miw_frag_load(int use, int dtype, int layout, int addr_space, int m, int n, int k,
+                  const void *addr, int64_t stride, void *frag, void *stream);
+
+/* store_d (src/device/cuda/wmma.jl:613-632; llvm_wmma_store_d_* :162-191). */
+int miw_frag_store(int dtype, int layout, int addr_space, int m, int n, int k,
+                   void *addr, const void *frag, int64_t stride, void *stream);
+
+/* fill_c (src/device/cuda/wmma.jl:654-667). */
+int miw_frag_fill(int dtype, float value, void *frag, void *stream);
+
+/* f.(frag, scalar) broadcasting (src/device/cuda/wmma.jl:678-716): out[i] =
+   scalar op in[i] in the fragment's element type, n_elems elements in total. */
+int miw_frag_map(int dtype, int op, float scalar, const void *in, void *out, size_t n_elems, void *stream);
+
+/* mma (src/device/cuda/wmma.jl:558-583; llvm_wmma_mma_* :222-257):
+   D = A*B + C on one 16x16x16 tile, A and B Float16, C and D independently
+   Float16 or Float32.  a_layout/b_layout are the layouts the fragments were
+   loaded with (part of the reference's fragment type); they are validated only:
+   the lane layout here does not depend on them. */
+int miw_frag_mma(int a_layout, int b_layout, int c_type, int d_type,
+                 const void *a_frag, const void *b_frag, const void *c_frag, void *d_frag, void *stream);
+
+typedef struct miw_mac_desc {
+    int m, n, k;                 /* must be 16,16,16 */
+    int a_layout, b_layout, c_layout, d_layout;
+    int c_type, d_type;
+    int use_c;                   /* 1: load_c (MAC); 0: fill_c(0) (MUL) */
+    int addr_space;              /* MIW_AS_* for every operand */
+    float alpha, beta;           /* a_frag = alpha .* a_frag (rounded to Float16),
+                                    c_frag = beta .* c_frag (in c_type) */
+    int64_t lda, ldb, ldc, ldd;
+} miw_mac_desc;
+
+/* The whole kernel of examples/wmma/high-level.jl:30-44 and of
+   test/device/wmma.jl:212-231 fused in one launch: load_a, load_b,
+   load_c | fill_c(0), alpha .* a, beta .* c, mma, store_d. */
+int miw_wmma_mac(const miw_mac_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream);
+
+/* ------------------------------------------------------------------- GEMM -- */
+
+typedef struct miw_gemm_desc {
+    int64_t m, n, k;
+    int64_t lda, ldb, ldc, ldd;          /* leading dimensions in elements */
+    int a_layout, b_layout, c_layout, d_layout;
+    int c_type, d_type;                  /* A and B are Float16 */
+    int acc_type;                        /* MIW_F32: fp32 accumulate.  MIW_F16: the
+                                            running sum is rounded to Float16 after
+                                            every acc_chunk k-values (needs c_type =
+                                            d_type = MIW_F16) */
+    int acc_chunk;                       /* 0 = variant's default */
+    float alpha, beta;
+    int use_c;                           /* 0: C is never read (fill_c(0)) */
+    int64_t batch;                       /* >= 1 */
+    int64_t stride_a, stride_b, stride_c, stride_d; /* elements between problems */
+    int variant;                         /* 0 = pick; see miw_gemm_variant_* */
+} miw_gemm_desc;
+
+/* D = alpha*A*B + beta*C, the chain of mma calls the reference describes
+   (docs/src/device/wmma.md:51-52) carried over the whole K extent.  M, N, K
+   must be multiples of 16; the LDS-tiled variants need multiples of their tile
+   (otherwise the fragment-op variant is used). */
+int miw_gemm(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream);
+
+/* Enumerate kernel variants (variant ids are 1..count). */
+int miw_gemm_variant_count(void);
+typedef struct miw_gemm_variant_info {
+    char name[64];
+    int block_m, block_n, block_k;
+    int waves_m, waves_n;
+    int stages;
+    int lds_bytes;
+    int fragment_ops;   /* 1: built from load_a/load_b/mma on global memory, no LDS */
+} miw_gemm_variant_info;
+int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
+/* Variant miw_gemm would pick for this descriptor. */
+int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant);
+/* acc_chunk miw_gemm would use for this descriptor (fp16 accumulate only). */
+int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk);
+
+/* warmup untimed launches, then iters launches each bracketed by HIP events on
+   `stream`; ms_each[i] receives launch i's duration in milliseconds. */
+int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D,
+                   void *stream, int warmup, int iters, float *ms_each);
+
+/* Register-resident back-to-back v_mfma_f32_16x16x32_f16 on every CU (the idea
+   of examples/peakflops.jl): measured TFLOP/s of the matrix cores alone. */
+int miw_mfma_peak_probe(int iters, double *tflops, void *stream);
+
+/* Plain device copy kernel (16 B per lane), used to calibrate HBM counters. */
+int miw_copy_probe(void *dst, const void *src, size_t bytes, void *stream);
+
+/* ----------------------------------------------------------- generic launch */
+/* @cuda threads= blocks= shmem= stream= f(args...) (src/execution.jl:45-114)
+   and cufunction / HostKernel (:205-219, :290-297) for the kernels compiled into
+   this library: look a kernel up by name, query its attributes
+   (registers/memory/maxthreads, :227-266), launch it with raw argument slots. */
+int miw_kernel_count(void);
+int miw_kernel_name(int index, char *buf, size_t buflen);
+int miw_kernel_lookup(const char *name, void **kernel);
+
+typedef struct miw_kernel_attributes {
+    int num_regs;
+    int max_threads_per_block;
+    size_t static_shared_bytes;
+    size_t local_bytes;
+    size_t const_bytes;
+} miw_kernel_attributes;
+int miw_kernel_attributes_get(void *kernel, miw_kernel_attributes *out);
+/* config= occupancy callback of @cuda (src/execution.jl:59-63):
+   hipOccupancyMaxPotentialBlockSize for this kernel. */
+int miw_kernel_occupancy(void *kernel, size_t dynamic_shmem, int *min_grid, int *block);
+int miw_launch(void *kernel, const unsigned grid[3], const unsigned block[3], unsigned shmem,
+               void *stream, void **args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIWMMA_H */
