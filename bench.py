@@ -1,0 +1,178 @@
+"""Benchmark of the hot path: fp16 -> fp32 GEMM D = A*B + C, M = N = K = 4096, column-major,
+one MI355X.  Prints one JSON line (TFLOP/s, roofline against the dense fp16 MFMA peak, and a CPU
+baseline timed on this host).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--variant V] [--no-cpu]
+
+A step is one GEMM launch on inputs already resident in HBM.  Each launch is bracketed by HIP
+events on the launch stream inside the library (miw_gemm_bench); `value` comes from the wall
+clock around the K steps (synchronised on both sides), `roofline.achieved` from the mean event
+duration of the same launches.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_F16_DENSE_TFLOPS = 2500.0   # MI355X published dense fp16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+CONFIGS = {
+    # name: (M, N, K, batch, a_layout, b_layout, c/d/acc type, description)
+    "c2": dict(M=4096, N=4096, K=4096, batch=1, a="col", b="col", half=False,
+               workload="gemm f16->f32 4096x4096x4096 column-major, D = A*B + C"),
+    "c3": dict(M=2048, N=2048, K=2048, batch=1, a="col", b="col", half=True,
+               workload="gemm all-f16 fp16-accumulate 2048x2048x2048 column-major"),
+    "c4": dict(M=8192, N=1024, K=4096, batch=1, a="row", b="col", half=False,
+               workload="gemm f16->f32 8192x1024x4096, A row-major, B column-major, C = 0"),
+    "c5": dict(M=128, N=128, K=128, batch=512, a="col", b="col", half=False,
+               workload="strided-batched gemm f16->f32 512 x 128x128x128 column-major"),
+}
+
+
+def cpu_baseline(orc, M, N, K, batch, budget_s=20.0):
+    """OpenBLAS sgemm through numpy on Float32 copies of the fp16 inputs, + C: the stand-in for
+    Julia's LinearAlgebra.mul! (Julia is not installed here).  Bounded to ~budget_s seconds."""
+    try:
+        from threadpoolctl import threadpool_info
+        info = [i for i in threadpool_info() if i.get("user_api") == "blas"]
+        threads = int(info[0]["num_threads"]) if info else (os.cpu_count() or 1)
+        blas = info[0].get("internal_api", "blas") if info else "blas"
+    except Exception:  # noqa: BLE001
+        threads, blas = (os.cpu_count() or 1), "blas"
+    nb = min(batch, 64)
+    a = orc.np_fill_uniform(nb * M * K, 11, -1.0, 1.0, np.float32).reshape(nb, K, M)
+    b = orc.np_fill_uniform(nb * K * N, 12, -1.0, 1.0, np.float32).reshape(nb, N, K)
+    c = orc.np_fill_uniform(nb * M * N, 13, -1.0, 1.0, np.float32).reshape(nb, N, M)
+    # column-major operands: D^T = B^T A^T in numpy's row-major view
+    def once():
+        d = np.matmul(b, a)
+        d += c
+        return d
+    once()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 7):
+        t0 = time.perf_counter()
+        once()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() > t_end and len(times) >= 3:
+            break
+    t = float(np.median(times))
+    return {
+        "value": 2.0 * M * N * K * nb / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"{len(times)} runs of the full {M}x{N}x{K}" + (f" x{nb} of {batch} problems" if batch > 1 else "")
+                  + f" sgemm + C on Float32 copies ({blas} via numpy, {threads} threads; not Julia mul!), median",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path runs on a single MI355X and nothing here shards it "
+              "(--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    from __graft_entry__ import load_package
+    from oracle import oracle as orc
+    m = load_package()
+    m.init(0)
+    info = m.device_info()
+    W, G = m.WMMA, m.GEMM
+    cfg = CONFIGS[args.config]
+    M, N, K, batch = cfg["M"], cfg["N"], cfg["K"], cfg["batch"]
+    half = cfg["half"]
+    ct = np.float16 if half else np.float32
+    lay = {"col": W.ColMajor, "row": W.RowMajor}
+
+    lo, hi, clo, chi = (-0.5, 0.5, -0.1, 0.1) if half else (-1.0, 1.0, -1.0, 1.0)
+    if args.config == "c4":
+        A = orc.np_fill_normal(batch * M * K, 3, 0.02, np.float16)
+        B = orc.np_fill_normal(batch * K * N, 1003, 0.02, np.float16)
+        C = np.zeros(batch * M * N, dtype=ct)
+    else:
+        A = orc.np_fill_uniform(batch * M * K, 1, lo, hi, np.float16)
+        B = orc.np_fill_uniform(batch * K * N, 1001, lo, hi, np.float16)
+        C = orc.np_fill_uniform(batch * M * N, 2001, clo, chi, ct)
+    dA, dB, dC = m.DeviceArray(A), m.DeviceArray(B), m.DeviceArray(C)
+    dD = m.DeviceArray.undef(ct, batch * M * N)
+    desc = G.make_desc(M, N, K, a_layout=lay[cfg["a"]], b_layout=lay[cfg["b"]], c_type=ct, d_type=ct,
+                       acc_type=ct, batch=batch, variant=args.variant)
+    variant = args.variant or G.pick_variant(desc)
+    vinfo = G.variants()[variant - 1]
+
+    # warm-up launches, then exactly `steps` launches between two synchronisations
+    if args.warmup:
+        G.gemm_bench(dA, dB, dC, dD, desc, warmup=0, iters=args.warmup)
+    m.synchronize()
+    t0 = time.perf_counter()
+    ms = G.gemm_bench(dA, dB, dC, dD, desc, warmup=0, iters=args.steps)
+    m.synchronize()
+    wall = time.perf_counter() - t0
+
+    flops = 2.0 * M * N * K * batch
+    gdesc = orc.GemmDesc(M=M, N=N, K=K, batch=batch, c_type=orc.F16 if half else orc.F32,
+                         d_type=orc.F16 if half else orc.F32)
+    abytes = gdesc.algorithmic_bytes()
+    ms_per_step = wall * 1e3 / args.steps
+    value = flops / (wall / args.steps) / 1e12
+    kernel_ms = float(np.mean(ms))
+
+    # correctness of what was just timed (sampled rows against float64)
+    D = dD.to_host()
+    g = orc.GemmDesc(M=M, N=N, K=K, batch=batch, a_layout=orc.ROW if cfg["a"] == "row" else orc.COL,
+                     b_layout=orc.ROW if cfg["b"] == "row" else orc.COL, c_type=gdesc.c_type, d_type=gdesc.d_type)
+    rows = np.arange(0, M, max(M // 64, 1))
+    ref = orc.np_gemm_rows_f64(g, A, B, C, rows)
+    got = orc.np_logical(g, D, "d")[rows, :]
+    err = float(np.abs(got - ref).max() / np.abs(ref).max())
+
+    if args.config == "c5":
+        roof = {"bound": "hbm", "achieved": abytes / (kernel_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s"}
+    else:
+        roof = {"bound": "mfma", "achieved": flops / (kernel_ms * 1e-3) / 1e12, "peak": PEAK_F16_DENSE_TFLOPS,
+                "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["kernel"] = "k_gemm_tiled<%s>" % vinfo["name"]
+    roof["kernel_ms_mean"] = kernel_ms
+    roof["kernel_ms_min"] = float(np.min(ms))
+
+    out = {
+        "metric": "TFLOP/s fp16->fp32 GEMM 4096^3 on 1xMI355X; % of fp16 MFMA peak" if args.config == "c2"
+                  else "TFLOP/s " + cfg["workload"],
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 in, f16 accumulate" if half else "f16 in, f32 accumulate", "data": "synthetic",
+        "config": {"workload": cfg["workload"], "variant": vinfo["name"], "batch": batch,
+                   "algorithmic_flop": flops, "algorithmic_bytes": abytes,
+                   "normalized_error_sampled": err, "tolerance": 1e-2 if half else 1e-3,
+                   "pct_of_fp16_dense_peak": 100.0 * value / PEAK_F16_DENSE_TFLOPS,
+                   "device": {"arch": info["arch"], "cus": info["cu_count"], "clock_mhz": info["clock_mhz"],
+                              "nominal_peak_tflops": info["peak_f16_tflops"]}},
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(orc, M, N, K, batch)
+    print(json.dumps(out))
+    tol = 1e-2 if half else 1e-3
+    if not err <= tol:
+        print(f"bench: result outside tolerance: {err} > {tol}", file=sys.stderr)
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

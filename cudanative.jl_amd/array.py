@@ -48,6 +48,20 @@ class DevicePtr:
             return self.addr - other.addr
         return DevicePtr(self.eltype, self.addr - int(other), self.addrspace, self._owner)
 
+    __radd__ = __add__
+
+    def convert(self, eltype=None, addrspace=None):
+        """convert(DevicePtr{T,A}, p): allowed within one address space and to or from
+        Generic; anything else is an ArgumentError (src/device/pointer.jl:85-97).
+        addrspace=None keeps the source's."""
+        eltype = self.eltype if eltype is None else eltype
+        if addrspace is None or addrspace == self.addrspace or AS.Generic in (addrspace, self.addrspace):
+            return self.unsafe_convert(eltype, self.addrspace if addrspace is None else addrspace)
+        raise ValueError("cannot convert between incompatible device pointer types")
+
+    def unsafe_convert(self, eltype, addrspace):
+        return DevicePtr(eltype, self.addr, addrspace, self._owner)
+
     def __eq__(self, other):
         return isinstance(other, DevicePtr) and self.addr == other.addr and self.addrspace == other.addrspace
 

@@ -406,6 +406,7 @@ int miwo_gemm_f16acc(const miwo_gemm_desc *g, int64_t kc, const uint16_t *A, con
 double miwo_normalized_error(const miwo_gemm_desc *g, const void *D, const double *dref)
 {
     double maxdiff = 0.0, maxref = 0.0;
+    int saw_nan = 0;
     size_t per = (size_t)g->M * (size_t)g->N;
     for (int64_t bt = 0; bt < (g->batch > 0 ? g->batch : 1); bt++) {
         const char *Db = (const char *)D + (size_t)(bt * g->stride_d) * (g->d_type == MIWO_F16 ? 2 : 4);
@@ -414,9 +415,11 @@ double miwo_normalized_error(const miwo_gemm_desc *g, const void *D, const doubl
                 double r = dref[(size_t)bt * per + (size_t)(i + j * g->M)];
                 double v = get_elem(Db, g->d_type, idx2(g->d_layout, (size_t)i, (size_t)j, (size_t)g->ldd));
                 double df = fabs(v - r);
-                if (!(df <= maxdiff)) maxdiff = df; /* NaN propagates */
+                if (df != df) saw_nan = 1;
+                else if (df > maxdiff) maxdiff = df;
                 if (fabs(r) > maxref) maxref = fabs(r);
             }
     }
+    if (saw_nan) return NAN;
     return maxref > 0.0 ? maxdiff / maxref : maxdiff;
 }

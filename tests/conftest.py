@@ -1,0 +1,52 @@
+import importlib.util
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG_DIR = os.path.join(ROOT, "cudanative.jl_amd")
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def load_package():
+    """Import the package directory `cudanative.jl_amd` under the module name cudanative_jl_amd."""
+    name = "cudanative_jl_amd"
+    if name in sys.modules:
+        return sys.modules[name]
+    if not os.path.exists(os.path.join(PKG_DIR, "libmiwmma.so")):
+        # nothing built yet: build once (hipcc cross-compiles without a GPU)
+        spec_b = importlib.util.spec_from_file_location("_miw_build", os.path.join(PKG_DIR, "build.py"))
+        b = importlib.util.module_from_spec(spec_b)
+        spec_b.loader.exec_module(b)
+        b.build()
+    spec = importlib.util.spec_from_file_location(name, os.path.join(PKG_DIR, "__init__.py"),
+                                                  submodule_search_locations=[PKG_DIR])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def miw():
+    return load_package()
+
+
+@pytest.fixture(scope="session")
+def gpu(miw):
+    """Initialised library on device 0.  GPU tests fail (not skip) when the HIP path cannot run."""
+    miw.init(0)
+    return miw
+
+
+@pytest.fixture(scope="session")
+def orc():
+    from oracle import oracle
+    oracle.lib()
+    return oracle

@@ -1,0 +1,329 @@
+"""GPU parity tests of the tiled GEMM D = alpha*A*B + beta*C, through the C ABI,
+against the CPU oracle (exact fp64 reference and the fp16-accumulate model)."""
+import itertools
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+F16, F32 = np.float16, np.float32
+
+# tolerances of BASELINE's north star: max|D - Dref| / max|Dref|
+TOL_F32ACC = 1e-3
+TOL_F16ACC = 1e-2
+# what fp32 accumulation actually achieves; a wrong tile or a dropped k-slice is ~1e-1
+TIGHT_F32 = 2e-6
+
+
+def _W(gpu, code):
+    return gpu.WMMA.ColMajor if code == 1 else gpu.WMMA.RowMajor
+
+
+def _run(gpu, orc, g, A, B, C, variant=0, acc_type=F32, acc_chunk=0, prefill=None):
+    """Run miw_gemm for oracle descriptor g on host buffers; returns D as a host buffer."""
+    g = g.resolved()
+    nb = max(g.batch, 1)
+    dA, dB = gpu.DeviceArray(A), gpu.DeviceArray(B)
+    dC = gpu.DeviceArray(C) if C is not None else None
+    dt = orc.np_dtype(g.d_type)
+    D0 = np.full(g.stride_d * nb, np.nan if prefill is None else prefill, dtype=dt)
+    dD = gpu.DeviceArray(D0)
+    desc = gpu.GEMM.make_desc(g.M, g.N, g.K, a_layout=_W(gpu, g.a_layout), b_layout=_W(gpu, g.b_layout),
+                              c_layout=_W(gpu, g.c_layout), d_layout=_W(gpu, g.d_layout),
+                              c_type=orc.np_dtype(g.c_type), d_type=dt, acc_type=acc_type, acc_chunk=acc_chunk,
+                              alpha=g.alpha, beta=g.beta, use_c=bool(g.use_c), batch=nb, lda=g.lda, ldb=g.ldb,
+                              ldc=g.ldc, ldd=g.ldd, stride_a=g.stride_a, stride_b=g.stride_b, stride_c=g.stride_c,
+                              stride_d=g.stride_d, variant=variant)
+    gpu.GEMM.gemm(dA, dB, dC, dD, desc)
+    gpu.synchronize()
+    return dD.to_host()
+
+
+def _inputs(orc, g, seed, ints=False, lo=-1.0, hi=1.0, clo=-1.0, chi=1.0):
+    g = g.resolved()
+    nb = max(g.batch, 1)
+    ct = orc.np_dtype(g.c_type)
+    if ints:
+        rng = np.random.default_rng(seed)
+        return (rng.integers(-3, 4, g.stride_a * nb).astype(F16), rng.integers(-3, 4, g.stride_b * nb).astype(F16),
+                rng.integers(-3, 4, g.stride_c * nb).astype(ct))
+    return (orc.np_fill_uniform(g.stride_a * nb, seed, lo, hi, F16),
+            orc.np_fill_uniform(g.stride_b * nb, seed + 1000, lo, hi, F16),
+            orc.np_fill_uniform(g.stride_c * nb, seed + 2000, clo, chi, ct))
+
+
+def _variants(gpu):
+    return gpu.GEMM.variants()
+
+
+def _tile_multiple(v, mult=(1, 1, 2)):
+    bm, bn, bk = v["block"]
+    return bm * mult[0], bn * mult[1], bk * mult[2]
+
+
+# ------------------------------------------------------------- exactness ----------
+
+@pytest.mark.parametrize("al,bl,dl", itertools.product((0, 1), repeat=3))
+def test_every_variant_exact_on_integer_inputs(gpu, orc, al, bl, dl):
+    """Small-integer inputs: every partial sum is exact, so any tiling must reproduce the oracle
+    bit for bit; catches a wrong index, a transposed operand, a missed k-slice."""
+    for v in _variants(gpu):
+        big = max(v["block"][:2])   # divisible by both tile extents, whichever dimension of D is contiguous
+        M, N, K = (48, 80, 96) if v["fragment_ops"] else (2 * big, big, 3 * v["block"][2])
+        g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl)
+        A, B, C = _inputs(orc, g, 100 + v["id"], ints=True)
+        D = _run(gpu, orc, g, A, B, C, variant=v["id"])
+        assert np.array_equal(D, orc.gemm(g, A, B, C)), (v["name"], al, bl, dl)
+
+
+def test_identity_and_ones(gpu, orc):
+    g = orc.GemmDesc(M=256, N=256, K=256)
+    _, B, C = _inputs(orc, g, 3)
+    eye = orc.to_storage(np.eye(256, dtype=F16), orc.COL)
+    D = _run(gpu, orc, g, eye, B, C)                     # A = I  =>  D = B + C exactly (fp32)
+    assert np.array_equal(D, (B.astype(F32) + C))
+    ones = np.ones(256 * 256, dtype=F16)
+    D = _run(gpu, orc, g, ones, ones, C)                 # all ones  =>  K + C
+    assert np.array_equal(D, (256 + C).astype(F32))
+
+
+# ------------------------------------------------------------- tolerance ----------
+
+@pytest.mark.parametrize("ct,dt", itertools.product((0, 1), repeat=2))
+def test_random_inputs_all_type_combinations(gpu, orc, ct, dt):
+    for v in _variants(gpu):
+        M, N, K = (64, 48, 208) if v["fragment_ops"] else _tile_multiple(v, (1, 1, 4))
+        g = orc.GemmDesc(M=M, N=N, K=K, c_type=ct, d_type=dt, alpha=0.75, beta=-1.25, a_layout=orc.ROW)
+        A, B, C = _inputs(orc, g, 7 * v["id"] + ct * 2 + dt)
+        D = _run(gpu, orc, g, A, B, C, variant=v["id"])
+        err = orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C))
+        assert err <= TOL_F32ACC
+        assert err <= (TIGHT_F32 if dt == orc.F32 else 6e-4), (v["name"], err)   # half output: 2^-11 relative
+
+
+def test_tiled_variants_agree_bitwise(gpu, orc):
+    """All LDS-tiled variants feed the same MFMA the same k-order per output element:
+    fp32 results are bit-identical across tile shapes (a staging or pipelining bug would differ)."""
+    g = orc.GemmDesc(M=512, N=512, K=512, b_layout=orc.ROW)
+    A, B, C = _inputs(orc, g, 21)
+    outs = [_run(gpu, orc, g, A, B, C, variant=v["id"]) for v in _variants(gpu) if not v["fragment_ops"]]
+    for o in outs[1:]:
+        assert np.array_equal(o.view(np.uint32), outs[0].view(np.uint32))
+    # twice the same launch: deterministic
+    assert np.array_equal(_run(gpu, orc, g, A, B, C, variant=1).view(np.uint32), outs[0].view(np.uint32))
+
+
+def test_ragged_sizes_fall_back_to_fragment_ops(gpu, orc):
+    # multiples of 16 that no LDS tile divides, padded leading dimensions, odd batch strides
+    g = orc.GemmDesc(M=80, N=112, K=176, lda=88, ldb=200, ldc=96, ldd=104, batch=3,
+                     stride_a=88 * 176 + 8, stride_b=200 * 112 + 24, stride_c=96 * 112, stride_d=104 * 112 + 40)
+    assert gpu.GEMM.variants()[gpu.GEMM.pick_variant(gpu.GEMM.make_desc(80, 112, 176)) - 1]["fragment_ops"]
+    A, B, C = _inputs(orc, g, 31)
+    D = _run(gpu, orc, g, A, B, C, prefill=-5.0)
+    assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+    # padding between columns and between batches is never written
+    gr = g.resolved()
+    Dm = D.reshape(-1)
+    for bt in range(3):
+        blk = Dm[bt * gr.stride_d: bt * gr.stride_d + 104 * 112].reshape(112, 104)
+        assert np.all(blk[:, 80:] == -5.0)
+        assert np.all(Dm[bt * gr.stride_d + 104 * 112:(bt + 1) * gr.stride_d] == -5.0)
+
+
+def test_tiled_with_padded_leading_dimensions_and_batch(gpu, orc):
+    g = orc.GemmDesc(M=128, N=128, K=192, lda=136, ldb=200, ldc=132, ldd=144, batch=5, a_layout=orc.COL, b_layout=orc.COL)
+    A, B, C = _inputs(orc, g, 41)
+    v = gpu.GEMM.pick_variant(gpu.GEMM.make_desc(128, 128, 192, batch=5, lda=136, ldb=200, ldc=132, ldd=144))
+    assert not gpu.GEMM.variants()[v - 1]["fragment_ops"]
+    D = _run(gpu, orc, g, A, B, C, prefill=9.0)
+    assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+    gr = g.resolved()
+    blk = D[: gr.stride_d].reshape(128, 144)
+    assert np.all(blk[:, 128:] == 9.0)
+    # batched == loop of single problems, bit for bit
+    for bt in (0, 4):
+        g1 = orc.GemmDesc(**{**g.__dict__, "batch": 1})
+        D1 = _run(gpu, orc, g1, A[bt * gr.stride_a:(bt + 1) * gr.stride_a], B[bt * gr.stride_b:(bt + 1) * gr.stride_b],
+                  C[bt * gr.stride_c:(bt + 1) * gr.stride_c], variant=v, prefill=9.0)
+        assert np.array_equal(D1.view(np.uint32), D[bt * gr.stride_d:(bt + 1) * gr.stride_d].view(np.uint32))
+
+
+def test_mul_path_never_reads_c(gpu, orc):
+    # use_c = 0 is fill_c(0): C may be NULL, beta is ignored, D is completely overwritten (it starts as NaN)
+    for variant in (0, len(_variants(gpu))):
+        g = orc.GemmDesc(M=256, N=128, K=128, use_c=0, beta=123.0, alpha=2.0, a_layout=orc.ROW, b_layout=orc.ROW)
+        A, B, _ = _inputs(orc, g, 51)
+        D = _run(gpu, orc, g, A, B, None, variant=variant)
+        assert not np.isnan(D).any()
+        assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, None)) <= TIGHT_F32
+
+
+def test_c_layout_differs_from_d_layout(gpu, orc):
+    for cl, dl in ((0, 1), (1, 0)):
+        g = orc.GemmDesc(M=256, N=256, K=64, c_layout=cl, d_layout=dl, beta=0.5)
+        A, B, C = _inputs(orc, g, 61)
+        D = _run(gpu, orc, g, A, B, C)
+        assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+
+
+def test_minimal_and_single_tile_shapes(gpu, orc):
+    for M, N, K in ((16, 16, 16), (64, 64, 64), (16, 256, 16), (256, 16, 1024)):
+        g = orc.GemmDesc(M=M, N=N, K=K)
+        A, B, C = _inputs(orc, g, M + N + K)
+        D = _run(gpu, orc, g, A, B, C)
+        assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+
+
+def test_golden_fixtures(gpu, orc):
+    from test_golden import SMALL
+    z = np.load(os.path.join(GOLD, "small_gemms.npz"))
+    for name, kw in SMALL.items():
+        g = orc.GemmDesc(**kw)
+        D = _run(gpu, orc, g, z[name + "_A"], z[name + "_B"], z[name + "_C"])
+        want = z[name + "_D"]
+        if g.d_type == orc.F32:
+            assert np.abs(D.astype(np.float64) - want.astype(np.float64)).max() <= 1e-5, name
+        else:  # at most one half ulp apart (fp32 sum rounded vs exact sum rounded)
+            assert np.abs(D.astype(np.float64) - want.astype(np.float64)).max() <= 2.0 ** -10 * np.abs(want).max(), name
+
+
+# ------------------------------------------------------------- fp16 accumulate ----
+
+def _assert_matches_model(got, model, min_equal=0.97):
+    """fp16-accumulate result vs the oracle's chunked model.  Both round at the same points; the
+    GPU's fp32 sum inside a chunk can differ from the exact chunk sum by an fp32 ulp, which flips a
+    half rounding only near a tie.  A flipped intermediate stays one half-ulp *of that intermediate*
+    off, so the bound is an ulp at the largest magnitude, and almost every element must be equal."""
+    got = np.asarray(got, dtype=np.float64)
+    model = np.asarray(model, dtype=np.float64)
+    diff = np.abs(got - model)
+    bound = 2.0 ** -9 * max(np.abs(model).max(), 1.0)
+    frac = float(np.mean(diff == 0))
+    assert diff.max() <= bound and frac > min_equal, (diff.max(), bound, frac)
+
+
+def test_f16acc_matches_the_chunked_model(gpu, orc):
+    z = np.load(os.path.join(GOLD, "small_gemms.npz"))
+    g = orc.GemmDesc(M=64, N=64, K=256, c_type=orc.F16, d_type=orc.F16)
+    A, B, C = z["h_A"], z["h_B"], z["h_C"]
+    ref = orc.gemm_f64(g, A, B, C)
+    nv = len(_variants(gpu))
+    for variant, kc in ((nv, 16), (nv - 1, 64)):          # fragment ops round every 16, the 64x64 tile every 64
+        desc = gpu.GEMM.make_desc(64, 64, 256, c_type=F16, d_type=F16, acc_type=F16, variant=variant)
+        assert gpu.GEMM.acc_chunk(desc) == kc
+        D = _run(gpu, orc, g, A, B, C, variant=variant, acc_type=F16)
+        assert orc.normalized_error(g, D, ref) <= TOL_F16ACC
+        model = z[f"h_D_kc{kc}"]
+        _assert_matches_model(D, model)
+        # and it is NOT the unchunked result: the model with a different chunk differs visibly
+        other = z[f"h_D_kc{80 - kc}"]
+        assert np.mean(D == other) < np.mean(D == model)
+
+
+def test_f16acc_exact_on_integers_all_variants(gpu, orc):
+    for v in _variants(gpu):
+        M, N, K = (48, 32, 64) if v["fragment_ops"] else _tile_multiple(v, (1, 1, 2))
+        g = orc.GemmDesc(M=M, N=N, K=K, c_type=orc.F16, d_type=orc.F16)
+        A, B, C = _inputs(orc, g, 71, ints=True)          # |sums| <= 9*K + 3 < 2048: exact in half
+        D = _run(gpu, orc, g, A, B, C, variant=v["id"], acc_type=F16)
+        assert np.array_equal(D, orc.gemm_f16acc(g, 16, A, B, C)), v["name"]
+
+
+def test_f16acc_alpha_beta(gpu, orc):
+    # alpha != 1 is served by the fragment-op kernel (rounding every 16); beta scales the initial accumulator
+    g = orc.GemmDesc(M=64, N=64, K=128, c_type=orc.F16, d_type=orc.F16, alpha=0.5, beta=2.0)
+    A, B, C = _inputs(orc, g, 81, lo=-0.5, hi=0.5, clo=-0.1, chi=0.1)
+    desc = gpu.GEMM.make_desc(64, 64, 128, c_type=F16, d_type=F16, acc_type=F16, alpha=0.5, beta=2.0)
+    assert gpu.GEMM.variants()[gpu.GEMM.pick_variant(desc) - 1]["fragment_ops"]
+    D = _run(gpu, orc, g, A, B, C, acc_type=F16)
+    model = orc.gemm_f16acc(g, 16, A, B, C)
+    _assert_matches_model(D, model)
+    with pytest.raises(gpu.MIWError):                     # a tiled variant cannot honour alpha != 1 in fp16 accumulate
+        _run(gpu, orc, g, A, B, C, acc_type=F16, variant=len(_variants(gpu)) - 1)
+
+
+# ------------------------------------------------------------- BASELINE configs ---
+
+def _sampled_error(orc, g, A, B, C, D, rows, bt=0):
+    """normalized error over a sample of full rows of D (D_ref rows in float64 by numpy)."""
+    gr = g.resolved()
+    ref = orc.np_gemm_rows_f64(g, A, B, C, rows, bt)
+    got = orc.np_logical(g, D, "d", bt)[rows, :]
+    return float(np.abs(got - ref).max() / np.abs(ref).max())
+
+
+def test_config2_4096_cubed(gpu, orc):
+    """C2: 4096^3 column-major, fp16 in / fp32 accumulate, seeded.  Full D checked against float64."""
+    n = 4096
+    g = orc.GemmDesc(M=n, N=n, K=n)
+    A, B, C = _inputs(orc, g, 1)
+    D = _run(gpu, orc, g, A, B, C)
+    ref = orc.np_gemm_f64(g, A, B, C)
+    err = orc.np_normalized_error(g, D, ref)
+    assert err <= TOL_F32ACC and err <= TIGHT_F32
+    # size-independent property: D(A, B, C) - D(A, B, 0) == C up to fp32 rounding of the sum
+    D0 = _run(gpu, orc, orc.GemmDesc(M=n, N=n, K=n, use_c=0), A, B, None)
+    assert np.abs((D.astype(np.float64) - D0.astype(np.float64)) - C).max() <= 2.0 ** -22 * np.abs(D0).max()
+
+
+def test_config3_fp16_accumulate_2048(gpu, orc):
+    """C3: 2048^3 all Float16, fp16 accumulate; A, B in [-0.5, 0.5], C in [-0.1, 0.1]."""
+    n = 2048
+    g = orc.GemmDesc(M=n, N=n, K=n, c_type=orc.F16, d_type=orc.F16)
+    A, B, C = _inputs(orc, g, 2, lo=-0.5, hi=0.5, clo=-0.1, chi=0.1)
+    D = _run(gpu, orc, g, A, B, C, acc_type=F16)
+    assert np.isfinite(D.astype(F32)).all()
+    err = orc.np_normalized_error(g, D, orc.np_gemm_f64(g, A, B, C))
+    assert err <= TOL_F16ACC
+    rows = np.arange(0, n, 64)
+    gr = orc.GemmDesc(M=len(rows), N=n, K=n, c_type=orc.F16, d_type=orc.F16, a_layout=orc.ROW)
+    Ar = np.ascontiguousarray(orc.np_logical_rows(g, A, rows).astype(F16)).reshape(-1)
+    Cr = orc.to_storage(orc.np_logical(g, C, "c")[rows, :].astype(F16), orc.COL)
+    desc = gpu.GEMM.make_desc(n, n, n, c_type=F16, d_type=F16, acc_type=F16)
+    model = orc.np_logical(gr, orc.gemm_f16acc(gr, gpu.GEMM.acc_chunk(desc), Ar, B, Cr), "d")
+    got = orc.np_logical(g, D, "d")[rows, :]
+    _assert_matches_model(got, model, min_equal=0.9)
+
+
+def test_config4_rectangular_mixed_layout(gpu, orc):
+    """C4: M=8192, N=1024, K=4096; A row-major, B column-major, N(0, 0.02^2); C zeros."""
+    g = orc.GemmDesc(M=8192, N=1024, K=4096, a_layout=orc.ROW, b_layout=orc.COL)
+    gr = g.resolved()
+    A = orc.np_fill_normal(gr.stride_a, 3, 0.02, F16)
+    B = orc.np_fill_normal(gr.stride_b, 1003, 0.02, F16)
+    C = np.zeros(gr.stride_c, dtype=F32)
+    D = _run(gpu, orc, g, A, B, C)
+    err = orc.np_normalized_error(g, D, orc.np_gemm_f64(g, A, B, C))
+    assert err <= TOL_F32ACC and err <= TIGHT_F32
+    # C = 0 is the MUL path
+    D0 = _run(gpu, orc, orc.GemmDesc(**{**g.__dict__, "use_c": 0}), A, B, None)
+    assert np.array_equal(D.view(np.uint32), D0.view(np.uint32))
+
+
+def test_config5_strided_batched(gpu, orc):
+    """C5: 512 independent 128^3 problems, contiguous batch strides."""
+    g = orc.GemmDesc(M=128, N=128, K=128, batch=512)
+    A, B, C = _inputs(orc, g, 4)
+    D = _run(gpu, orc, g, A, B, C)
+    err = orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C))
+    assert err <= TOL_F32ACC and err <= TIGHT_F32
+    # checksum of checksums: sum over the batch of column sums, against numpy on the inputs
+    a = A.reshape(512, 128, 128).astype(np.float64)      # [bt][k][m]
+    b = B.reshape(512, 128, 128).astype(np.float64)      # [bt][n][k]
+    want = np.einsum("bk,bnk->n", a.sum(axis=2), b) + C.reshape(512, 128, 128).astype(np.float64).sum(axis=(0, 2))
+    got = D.reshape(512, 128, 128).astype(np.float64).sum(axis=(0, 2))
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-3)
+
+
+def test_bench_entry_reports_positive_times(gpu, orc):
+    g = orc.GemmDesc(M=256, N=256, K=256)
+    A, B, C = _inputs(orc, g, 9)
+    dA, dB, dC = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(C)
+    dD = gpu.DeviceArray.undef(F32, 256 * 256)
+    ms = gpu.GEMM.gemm_bench(dA, dB, dC, dD, gpu.GEMM.make_desc(256, 256, 256), warmup=2, iters=5)
+    assert ms.shape == (5,) and np.all(ms > 0) and np.all(ms < 50)
+    assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+    assert gpu.mfma_peak_tflops(2000) > 100

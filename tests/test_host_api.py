@@ -1,0 +1,220 @@
+"""Host-side logic that needs no GPU: the exact host tests of the reference
+(flatten/unflatten, fragment broadcasting, DevicePtr), argument validation of the
+C ABI, and that the shared library exports what include/miwmma.h declares."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- test/device/wmma.jl:156-176 -------------------------------------------------
+
+def test_flatten(miw):
+    W = miw.WMMA
+    F16 = W.Float16
+    assert W.flatten(5) == (5,)
+    assert W.flatten(5.0) == (5.0,)
+    assert W.flatten(W.VecElement(F16, 5)) == (F16(5),)
+    assert W.flatten(tuple(range(1, 9))) == tuple(range(1, 9))
+    assert W.flatten(tuple(W.VecElement(F16, i) for i in range(1, 9))) == tuple(F16(i) for i in range(1, 9))
+    assert W.flatten(tuple(tuple((i - 1) * 2 + j for j in (1, 2)) for i in range(1, 9))) == tuple(range(1, 17))
+    assert W.flatten(tuple(tuple(W.VecElement(F16, (i - 1) * 2 + j) for j in (1, 2)) for i in range(1, 9))) == \
+        tuple(F16(i) for i in range(1, 17))
+
+
+def test_unflatten(miw):
+    W = miw.WMMA
+    F16 = W.Float16
+    assert W.unflatten(np.int64, (5,)) == 5
+    assert W.unflatten(np.float64, (5.0,)) == 5.0
+    assert W.unflatten(W.VecElementType(F16), (F16(5),)) == W.VecElement(F16, 5)
+    assert W.unflatten(W.NTuple(8, np.int64), tuple(range(1, 9))) == tuple(range(1, 9))
+    assert W.unflatten(W.NTuple(8, W.VecElementType(F16)), tuple(F16(i) for i in range(1, 9))) == \
+        tuple(W.VecElement(F16, i) for i in range(1, 9))
+    assert W.unflatten(W.NTuple(8, W.NTuple(2, np.int64)), tuple(range(1, 17))) == \
+        tuple(tuple((i - 1) * 2 + j for j in (1, 2)) for i in range(1, 9))
+    assert W.unflatten(W.NTuple(8, W.NTuple(2, W.VecElementType(F16))), tuple(F16(i) for i in range(1, 17))) == \
+        tuple(tuple(W.VecElement(F16, (i - 1) * 2 + j) for j in (1, 2)) for i in range(1, 9))
+
+
+# ---- test/device/wmma.jl:180-184 -------------------------------------------------
+
+@pytest.mark.parametrize("sz", [1, 2, 5])
+@pytest.mark.parametrize("ty", [np.float16, np.float32])
+def test_fragment_broadcast_host(miw, sz, ty):
+    W = miw.WMMA
+    frag = W.Fragment(16, 16, 16, sz, ty, W.RowMajor, W.MatrixA, tuple(ty(i) for i in range(1, sz + 1)))
+    assert ty(5) * frag == W.Fragment(16, 16, 16, sz, ty, W.RowMajor, W.MatrixA, tuple(ty(5 * i) for i in range(1, sz + 1)))
+    assert ty(5) + frag == W.Fragment(16, 16, 16, sz, ty, W.RowMajor, W.MatrixA, tuple(ty(5 + i) for i in range(1, sz + 1)))
+    assert (ty(5) * frag).type_params() == frag.type_params()
+    assert frag[0] == ty(1) and frag[frag.lastindex()] == ty(sz) and frag.firstindex() == 0
+    assert ty(5) * frag != W.Fragment(16, 16, 16, sz, ty, W.ColMajor, W.MatrixA, tuple(ty(5 * i) for i in range(1, sz + 1)))
+
+
+# ---- test/pointer.jl:1-60 ----------------------------------------------------------
+
+def test_device_pointer(miw):
+    P, AS = miw.DevicePtr, miw.AS
+    ga = P(np.uint8, 0xDEADBEEF)
+    gla = P(np.uint8, 0xDEADBEEF, AS.Global)
+    la = P(np.uint8, 0xDEADBEEF, AS.Local)
+    gb = P(np.uint8, 0xCAFEBABE)
+    glb = P(np.uint8, 0xCAFEBABE, AS.Global)
+    gib = P(np.int64, 0xCAFEBABE)
+    glib = P(np.int64, 0xCAFEBABE, AS.Global)
+    assert ga.addrspace == AS.Generic and gla.addrspace == AS.Global and la.addrspace == AS.Local
+    assert glib.eltype == np.int64
+    assert ga != gla and ga != gib
+    assert int(ga) == 0xDEADBEEF
+    with pytest.raises(ValueError):
+        gla.convert(np.uint8, AS.Local)
+    assert ga.convert(np.uint8, AS.Generic) == ga
+    assert gla.convert(np.uint8, AS.Global) == gla
+    assert gla.unsafe_convert(np.uint8, AS.Local) == la
+    assert glib.convert(np.uint8, AS.Global) == glb
+    assert glib.convert(np.uint8, AS.Generic) == gb
+    assert gib.convert(np.uint8, AS.Global) == glb
+    assert glib.convert(np.uint8) == glb                      # unspecified: keeps the address space
+    assert (ga + 16).addr == 0xDEADBEEF + 16 and (16 + ga) == ga + 16 and (ga + 16) - ga == 16
+    assert (AS.Generic, AS.Global, AS.Shared, AS.Constant, AS.Local) == (0, 1, 3, 4, 5)
+
+
+# ---- Config / type rules -----------------------------------------------------------
+
+def test_config_and_invalid_arguments(miw):
+    W = miw.WMMA
+    conf = W.Config[16, 16, 16, W.Float32]
+    assert conf == W.Config(16, 16, 16, np.float32) and repr(conf) == "Config{16,16,16,float32}"
+    p16 = miw.DevicePtr(np.float16, 0x1000, miw.AS.Global)
+    p32 = miw.DevicePtr(np.float32, 0x1000, miw.AS.Global)
+    with pytest.raises(W.WMMAError, match=r"Invalid shape for WMMA: \(M, N, K\) = \(16, 16, 8\)"):
+        W.load_a(p16, 16, W.ColMajor, W.Config(16, 16, 8, W.Float32))
+    with pytest.raises(W.WMMAError, match="Invalid layout for WMMA"):
+        W.load_a(p16, 16, W.Unspecified, conf)
+    with pytest.raises(W.WMMAError, match="Invalid address space for WMMA"):
+        W.load_a(miw.DevicePtr(np.float16, 0x1000, miw.AS.Constant), 16, W.ColMajor, conf)
+    with pytest.raises(W.WMMAError, match="Invalid type float32 for matrix a"):
+        W.load_a(p32, 16, W.ColMajor, conf)
+    with pytest.raises(W.WMMAError, match="Invalid element type for WMMA"):
+        W.load_c(miw.DevicePtr(np.float64, 0x1000, miw.AS.Global), 16, W.ColMajor, conf)
+    with pytest.raises(W.WMMAError, match="Invalid element type for WMMA"):
+        W.fill_c(1.0, conf)
+    host = W.Fragment(16, 16, 16, 4, np.float16, W.ColMajor, W.MatrixA, (1, 2, 3, 4))
+    with pytest.raises(TypeError):
+        W.mma(host, host, host, conf)            # b is not a MatrixB
+    with pytest.raises(TypeError):
+        W.store_d(p16, W.Fragment(16, 16, 16, 4, np.float32, W.Unspecified, W.Accumulator, (1, 2, 3, 4)), 16,
+                  W.ColMajor, conf)               # eltype(addr) != eltype(d)
+    assert len(W.LOW_LEVEL_NAMES) == 52 and len(set(W.LOW_LEVEL_NAMES)) == 52
+    assert "llvm_wmma_load_a_col_m16n16k16_global_stride_f16" in W.LOW_LEVEL_NAMES
+    assert "llvm_wmma_mma_row_col_m16n16k16_f32_f16" in W.LOW_LEVEL_NAMES
+    assert "llvm_wmma_store_d_row_m16n16k16_shared_stride_f32" in W.LOW_LEVEL_NAMES
+    with pytest.raises(ValueError, match="Unsupported keyword argument 'cooperative'"):
+        miw.cuda(lambda: None, cooperative=True)
+
+
+# ---- C ABI -------------------------------------------------------------------------
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "miwmma.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(miw_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(miw):
+    names = _declared_functions()
+    assert len(names) >= 35
+    lib = ctypes.CDLL(miw._lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in miwmma.h but not exported"
+    assert sorted(miw._lib.SIGNATURES) == names
+
+
+def test_struct_sizes_match_header(miw):
+    # compile-free check of the ABI structs: sizes as a C compiler lays them out
+    L = miw._lib
+    assert ctypes.sizeof(L.MacDesc) == 13 * 4 + 4 + 4 * 8      # 13 ints/floats, pad, 4 int64
+    assert ctypes.sizeof(L.GemmDesc) == 7 * 8 + 11 * 4 + 4 + 5 * 8 + 8
+    assert ctypes.sizeof(L.GemmVariantInfo) == 64 + 8 * 4
+    assert ctypes.sizeof(L.DeviceInfo) == 128 + 64 + 7 * 4 + 4 + 2 * 8 + 8
+
+
+def test_abi_rejects_bad_arguments_without_touching_the_gpu(miw):
+    L = miw._lib
+    lib = L.load()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    p = (p + 15) & ~15
+    assert lib.miw_frag_load(L.MATRIX_A, L.F16, L.COL_MAJOR, L.AS_GLOBAL, 16, 16, 8, p, 16, p, None) == L.ERR_INVALID_SHAPE
+    assert "Invalid shape for WMMA: (M, N, K) = (16, 16, 8)" in L.last_error()
+    assert lib.miw_frag_load(L.MATRIX_A, L.F16, 7, L.AS_GLOBAL, 16, 16, 16, p, 16, p, None) == L.ERR_INVALID_LAYOUT
+    assert lib.miw_frag_load(L.MATRIX_A, L.F16, L.COL_MAJOR, 4, 16, 16, 16, p, 16, p, None) == L.ERR_INVALID_AS
+    assert lib.miw_frag_load(L.MATRIX_A, L.F32, L.COL_MAJOR, L.AS_GLOBAL, 16, 16, 16, p, 16, p, None) == L.ERR_INVALID_TYPE
+    assert "Invalid type Float32 for matrix a" in L.last_error()
+    assert lib.miw_frag_load(L.ACCUMULATOR, L.F32, L.COL_MAJOR, L.AS_GLOBAL, 16, 16, 16, None, 16, p, None) == L.ERR_NULL_POINTER
+    assert lib.miw_frag_load(L.ACCUMULATOR, L.F32, L.COL_MAJOR, L.AS_GLOBAL, 16, 16, 16, p + 2, 16, p, None) == L.ERR_MISALIGNED
+    assert lib.miw_frag_store(L.F32, L.COL_MAJOR, L.AS_GLOBAL, 16, 16, 16, p, p, 8, None) == L.ERR_INVALID_VALUE
+    assert lib.miw_frag_fill(9, 0.0, p, None) == L.ERR_INVALID_TYPE
+    assert lib.miw_frag_map(L.F16, 5, 1.0, p, p, 4, None) == L.ERR_INVALID_VALUE
+    assert lib.miw_frag_mma(L.COL_MAJOR, 3, L.F16, L.F16, p, p, p, p, None) == L.ERR_INVALID_LAYOUT
+    assert lib.miw_frag_elems_per_lane(L.ACCUMULATOR, L.F32) == 4
+    assert lib.miw_frag_image_bytes(L.MATRIX_A, L.F16) == 512 and lib.miw_frag_image_bytes(L.ACCUMULATOR, L.F32) == 1024
+
+    G = miw.GEMM
+    d = G.make_desc(100, 64, 64)
+    assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_SHAPE
+    d = G.make_desc(64, 64, 64, lda=32)
+    assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_VALUE
+    d = G.make_desc(64, 64, 64, c_type=np.float32, d_type=np.float16, acc_type=np.float16)
+    assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_TYPE
+    d = G.make_desc(64, 64, 64)
+    assert lib.miw_gemm(ctypes.byref(d), p, None, p, p, None) == L.ERR_NULL_POINTER
+    assert lib.miw_gemm(ctypes.byref(d), p + 1, p, p, p, None) == L.ERR_MISALIGNED
+    d = G.make_desc(64, 64, 64, variant=99)
+    assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_VALUE
+    d = G.make_desc(64, 64, 64, batch=0)
+    assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_VALUE
+    d = G.make_desc(80, 64, 64, variant=1)                     # not divisible by the 256x256 tile
+    assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_UNSUPPORTED
+    k = ctypes.c_void_p()
+    assert lib.miw_kernel_lookup(b"no_such_kernel", ctypes.byref(k)) == L.ERR_NOT_FOUND
+    assert lib.miw_launch(ctypes.c_void_p(0x1234), (ctypes.c_uint * 3)(1, 1, 1), (ctypes.c_uint * 3)(64, 1, 1), 0, None,
+                          None) == L.ERR_NOT_FOUND
+
+
+def test_variant_table_and_selection(miw):
+    G = miw.GEMM
+    vs = G.variants()
+    assert vs[-1]["fragment_ops"] and vs[-1]["name"] == "fragment_ops"
+    assert all(v["lds_bytes"] <= 160 * 1024 for v in vs)
+    assert all(v["lds_bytes"] == v["stages"] * (v["block"][0] + v["block"][1]) * v["block"][2] * 2 for v in vs[:-1])
+    by = {v["name"]: v["id"] for v in vs}
+    # 4096^3 fills 256 CUs with 256x256 tiles; small or odd shapes fall to smaller tiles / fragment ops
+    assert G.pick_variant(G.make_desc(4096, 4096, 4096)) == 1
+    assert vs[G.pick_variant(G.make_desc(128, 128, 128, batch=512)) - 1]["block"][:2] == (128, 128)
+    assert G.pick_variant(G.make_desc(48, 48, 48)) == by["fragment_ops"]
+    assert G.pick_variant(G.make_desc(64, 64, 80)) == by["fragment_ops"]
+    d = G.make_desc(2048, 2048, 2048, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
+    assert G.acc_chunk(d) == 64
+    d = G.make_desc(48, 48, 48, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
+    assert G.acc_chunk(d) == 16
+    names = miw.kernel_names()
+    assert "wmma_mac_f32_f32" in names and "gemm_tile256x256_w2x4" in names
+
+
+def test_no_device_errors_are_clean(miw):
+    # Without a GPU every device entry returns a HIP error code and a message (never crashes);
+    # with one, init succeeds.
+    import subprocess, sys
+    code = ("import sys; sys.path.insert(0, %r); from tests.conftest import load_package; m = load_package();\n"
+            "import ctypes; p = ctypes.c_void_p();\n"
+            "try:\n    m.init(0); print('ok')\n"
+            "except m.MIWError as e:\n    assert e.code > 0 and 'hip' in e.message.lower(), e; print('nodevice')\n") % ROOT
+    env = dict(os.environ, HIP_VISIBLE_DEVICES="-1", ROCR_VISIBLE_DEVICES="-1")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip() == "nodevice"
