@@ -4,10 +4,9 @@ baseline timed on this host).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--variant V] [--no-cpu]
 
-A step is one GEMM launch on inputs already resident in HBM.  Each launch is bracketed by HIP
-events on the launch stream inside the library (miw_gemm_bench); `value` comes from the wall
-clock around the K steps (synchronised on both sides), `roofline.achieved` from the mean event
-duration of the same launches.
+A step is one GEMM launch on inputs already resident in HBM.  `value` comes from the wall clock
+around K back-to-back launches (synchronised on both sides); `roofline.achieved` from the HIP-event
+time over the same K launches, recorded on the launch stream, divided by K.
 """
 import argparse
 import json
@@ -22,6 +21,13 @@ sys.path.insert(0, ROOT)
 
 PEAK_F16_DENSE_TFLOPS = 2500.0   # MI355X published dense fp16 MFMA peak
 PEAK_HBM_GBS = 8000.0
+# L2 <-> fabric bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs),
+# each scaled by what the counter reads for the library's copy kernel on 256 MiB; the summaries
+# and commands are under profiles/.  Configurations without a measurement report null.
+MEASURED_TRAFFIC_BYTES = {
+    "c2": int((257.3 + 73.0) * 2 ** 20),   # profiles/gemm_tiled_256x256_c2_4096cubed.md
+    "c5": int((64.1 + 32.0) * 2 ** 20),    # profiles/gemm_tiled_128x128_c5_batched128.md
+}
 
 CONFIGS = {
     # name: (M, N, K, batch, a_layout, b_layout, c/d/acc type, description)
@@ -80,6 +86,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="instead of the GEMM, launch the library's plain copy kernel on MIB MiB a few times "
+                         "(calibrates the FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path runs on a single MI355X and nothing here shards it "
@@ -90,6 +99,15 @@ def main():
     from oracle import oracle as orc
     m = load_package()
     m.init(0)
+    if args.copy_probe:
+        n = args.copy_probe << 20
+        src, dst = m.DeviceArray.undef(np.uint8, n), m.DeviceArray.undef(np.uint8, n)
+        src.fill_bytes(1)
+        for _ in range(5):
+            m._lib.check(m._lib.load().miw_copy_probe(dst.ptr, src.ptr, n, None))
+        m.synchronize()
+        print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "launches": 5}))
+        return
     info = m.device_info()
     W, G = m.WMMA, m.GEMM
     cfg = CONFIGS[args.config]
@@ -114,14 +132,27 @@ def main():
     variant = args.variant or G.pick_variant(desc)
     vinfo = G.variants()[variant - 1]
 
-    # warm-up launches, then exactly `steps` launches between two synchronisations
-    if args.warmup:
-        G.gemm_bench(dA, dB, dC, dD, desc, warmup=0, iters=args.warmup)
+    # warm-up launches, then exactly `steps` back-to-back launches between two synchronisations;
+    # one HIP event on the launch stream (the default stream) at each end of the timed region
+    import ctypes
+    lib = m._lib.load()
+    ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
+    m._lib.check(lib.miw_event_create(ctypes.byref(ev0)))
+    m._lib.check(lib.miw_event_create(ctypes.byref(ev1)))
+    for _ in range(args.warmup):
+        G.gemm(dA, dB, dC, dD, desc)
     m.synchronize()
     t0 = time.perf_counter()
-    ms = G.gemm_bench(dA, dB, dC, dD, desc, warmup=0, iters=args.steps)
+    m._lib.check(lib.miw_event_record(ev0, None))
+    for _ in range(args.steps):
+        G.gemm(dA, dB, dC, dD, desc)
+    m._lib.check(lib.miw_event_record(ev1, None))
     m.synchronize()
     wall = time.perf_counter() - t0
+    ev_ms = ctypes.c_float()
+    m._lib.check(lib.miw_event_elapsed_ms(ctypes.byref(ev_ms), ev0, ev1))
+    # outside the timed region: the same launches again, each bracketed by its own pair of events
+    ms = G.gemm_bench(dA, dB, dC, dD, desc, warmup=0, iters=min(args.steps, 50))
 
     flops = 2.0 * M * N * K * batch
     gdesc = orc.GemmDesc(M=M, N=N, K=K, batch=batch, c_type=orc.F16 if half else orc.F32,
@@ -129,7 +160,7 @@ def main():
     abytes = gdesc.algorithmic_bytes()
     ms_per_step = wall * 1e3 / args.steps
     value = flops / (wall / args.steps) / 1e12
-    kernel_ms = float(np.mean(ms))
+    kernel_ms = float(ev_ms.value) / args.steps   # mean launch duration over the timed region
 
     # correctness of what was just timed (sampled rows against float64)
     D = dD.to_host()
@@ -146,10 +177,11 @@ def main():
         roof = {"bound": "mfma", "achieved": flops / (kernel_ms * 1e-3) / 1e12, "peak": PEAK_F16_DENSE_TFLOPS,
                 "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.config) if not args.variant else None
     roof["kernel"] = "k_gemm_tiled<%s>" % vinfo["name"]
     roof["kernel_ms_mean"] = kernel_ms
-    roof["kernel_ms_min"] = float(np.min(ms))
+    roof["kernel_ms_median_single"] = float(np.median(ms))
+    roof["kernel_ms_min_single"] = float(np.min(ms))
 
     out = {
         "metric": "TFLOP/s fp16->fp32 GEMM 4096^3 on 1xMI355X; % of fp16 MFMA peak" if args.config == "c2"

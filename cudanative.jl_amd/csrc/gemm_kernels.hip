@@ -1,6 +1,6 @@
 // LDS-tiled mixed-precision GEMM for gfx950: D = alpha * A*B + beta * C with
 // Float16 A and B, fp32 accumulation in v_mfma_f32_16x16x32_f16 (optionally
-// rounded to Float16 after every K-tile: the fp16-accumulate variant).
+// rounded to Float16 every 64 k-values: the fp16-accumulate variant).
 //
 // It is the chain "D of one mma is C of the next" (CUDAnative.jl
 // docs/src/device/wmma.md:51-52) carried over K, with the fragment loads of
@@ -14,17 +14,26 @@
 // bytes per lane.  X is "K-major" when its k index is contiguous in memory
 // (A row-major / B column-major) and "I-major" otherwise; likewise Y.
 //
-// LDS tile layouts (K-tile = 64 k-values, 16-byte chunks):
-//   K-major operand, R rows : chunk (r, c) of row r (8 chunks of 8 k-values)
-//       sits at chunk index r*8 + (c ^ ((r >> 1) & 7)).  A lane reads its 8
-//       k-values for the MFMA with one ds_read_b128; the XOR spreads the 16
-//       rows of a fragment over all banks.
-//   I-major operand (k rows of R contiguous i) : stored as 128-byte blocks of
-//       4 k-values x 16 i, one block = what 16 lanes fetch with one
-//       ds_read_b64_tr_b16 (the LDS transpose read), which hands each lane
-//       4 consecutive k-values of its row.  Block (k4, i16) with
-//       k4 = 4a + 2mid + lo sits at block index ((2a + lo)*(R/16) + i16)*2 + mid,
-//       so the four 16-lane groups of one read hit alternating 128-byte halves.
+// Pipeline.  K is consumed in steps of 32 k-values (one MFMA k-step), fetched
+// in pairs: LDS holds two slots of 64 k-values.  While the matrix cores work
+// through the fragments of step s out of one register set, the fragments of
+// step s+1 are read from LDS into a second set (reads first, so that they have
+// landed long before the step ends), and the direct-to-LDS loads of the next
+// pair are in flight.  One s_barrier per pair publishes the pair that landed
+// and frees the slot of the pair that has been read.
+//
+// LDS slot layouts (16-byte chunks of 8 k-values or 8 i-values), chosen so that
+// every 8 consecutive lanes of a direct-to-LDS load fetch one full 128-byte
+// line and every fragment read is free of bank conflicts:
+//   K-major operand, R rows of 128 bytes: chunk (r, c), c = 0..7, sits at chunk
+//       index r*8 + (c ^ ((r >> 1) & 7)).  A lane reads its 8 k-values of a
+//       32-k step with one ds_read_b128.
+//   I-major operand (64 k-rows of R contiguous i): row pieces of 64 i (128 B)
+//       at chunk index ((i/64)*64 + k)*8 + (c ^ 2g(k)), c = 0..7,
+//       g(k) = ((k>>1)&1) | (((k>>3)&1)<<1).  A fragment is fetched with two
+//       ds_read_b64_tr_b16 (the LDS transpose read): 16 lanes pick up 4 k-rows
+//       x 16 i and each lane receives 4 consecutive k-values of its row; the
+//       XOR spreads the 16 row pieces of one read over all banks.
 //   Direct-to-LDS loads write lane-contiguous 1 KiB per wavefront instruction;
 //   the layouts above are produced by choosing which global chunk each lane
 //   fetches.
@@ -45,7 +54,9 @@ typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
 #define MIW_LDS __attribute__((address_space(3)))
 #define MIW_GLOBAL __attribute__((address_space(1)))
 
-constexpr int BK = 64;  // k-values per K-tile
+constexpr int BKS = 32;    // k-values per pipeline step (one MFMA k-step)
+constexpr int KGRAN = 64;  // k-values per LDS slot and K granularity of the kernel
+constexpr int NSLOT = 2;   // LDS slots
 
 struct tiled_params {
     const half_t *X;
@@ -61,14 +72,24 @@ struct tiled_params {
     int tiles_i, tiles_j, group_i;
 };
 
-// vmcnt(n) with expcnt/lgkmcnt left alone (gfx9 encoding).
-#define MIW_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+// s_waitcnt vmcnt(N) lgkmcnt(0); s_barrier.  The direct-to-LDS loads are issued
+// from inline assembly (the compiler's own wait-count pass would otherwise
+// serialise them with every LDS read of the other slot), so their completion is
+// tracked by hand: vmcnt(N) leaves the N youngest in flight.  The wait itself
+// is the compiler builtin, so that the compiler knows the LDS reads issued so
+// far have landed; the empty asm statements keep LDS reads and loads from
+// moving across the barrier.
+template <int N>
+__device__ inline void wait_loads_and_barrier()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 
 // One 16-byte-per-lane direct-to-LDS load: lane l fetches base + voff[l] and
-// the wavefront's 1 KiB lands at LDS byte lds_addr + 16*l.  Written as inline
-// assembly so that the compiler's wait-count pass does not serialise it with
-// the LDS reads of the other stage; completion is awaited explicitly with
-// MIW_WAIT_VMCNT before the barrier that publishes the tile.
+// the wavefront's 1 KiB lands at LDS byte lds_addr + 16*l.
 __device__ inline void lds_dma16(const void *base, unsigned voff, unsigned lds_addr)
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -77,78 +98,89 @@ __device__ inline void lds_dma16(const void *base, unsigned voff, unsigned lds_a
                  : "memory", "m0");
 }
 
-// ------------------------------------------------------------ tile loader --
-template <int R, bool KMAJOR, int NT>
-struct tile_loader {
-    static constexpr int CHUNKS = R * 8;
-    static constexpr int NLOAD = CHUNKS / NT;
-    static_assert(CHUNKS % NT == 0, "tile must divide over the workgroup");
+__device__ inline int i_major_swizzle(int k) { return ((k >> 1) & 1) | (((k >> 3) & 1) << 1); }
 
-    // Element offset, relative to the tile origin at k-tile 0, of the global
-    // chunk that lands in LDS chunk q.
-    __device__ static inline int source_offset(int q, int ld)
+// ------------------------------------------------------------ slot loader --
+// Fetches one slot (R rows/columns x 64 k-values) with NT threads.  Thread t
+// owns LDS chunks t, t + NT, t + 2 NT, ...; their global sources differ by
+// offsets that are the same for every thread, so one lane offset is kept and
+// the rest is scalar address arithmetic.
+template <int R, bool KMAJOR, int NT>
+struct slot_loader {
+    static constexpr int CHUNKS = R * KGRAN / 8;
+    static constexpr int NLOAD = CHUNKS / NT;
+    static_assert(CHUNKS % NT == 0 && (NT == 256 || NT == 512), "slot must divide over the workgroup");
+
+    // Byte offset, relative to the slot origin in global memory, of the chunk
+    // this thread fetches first.
+    __device__ static inline unsigned lane_offset(int tid, int ld)
     {
         if constexpr (KMAJOR) {
-            const int r = q >> 3, cpos = q & 7;
+            const int r = tid >> 3, cpos = tid & 7;
             const int c = cpos ^ ((r >> 1) & 7);
-            return r * ld + c * 8;
+            return 2u * (unsigned)(r * ld + c * 8);
         } else {
-            constexpr int R16 = R / 16;
-            const int b = q >> 3, kq = (q & 7) >> 1, hf = q & 1;
-            const int mid = b & 1, rest = b >> 1;
-            const int i16 = rest % R16, x = rest / R16;
-            const int k4 = 4 * (x >> 1) + 2 * mid + (x & 1);
-            return (4 * k4 + kq) * ld + 16 * i16 + 8 * hf;
+            const int k = (tid >> 3) & 63, cpos = tid & 7;  // tid / 512 == 0
+            const int c = cpos ^ (2 * i_major_swizzle(k));
+            return 2u * (unsigned)(k * ld + c * 8);
         }
     }
 
-    // Byte offsets of this thread's chunks.
-    __device__ static inline void offsets(int tid, int ld, unsigned (&off)[NLOAD])
+    // Element offset of load i relative to load 0 (uniform).
+    __device__ static inline long load_delta(int i, long ld)
     {
-#pragma unroll
-        for (int i = 0; i < NLOAD; i++) off[i] = 2u * (unsigned)source_offset(i * NT + tid, ld);
+        if constexpr (KMAJOR) {
+            return (long)i * (NT / 8) * ld;  // NT/8 rows further down
+        } else {
+            const int k = (i * (NT / 8)) & 63, iblk = (i * NT) / 512;
+            return (long)k * ld + iblk * 64;
+        }
     }
 
-    // base: uniform global address of the tile origin; lds_wave: this
+    // base: uniform global address of the slot origin; lds_wave: this
     // wavefront's first destination byte for load 0 (uniform).
-    __device__ static inline void issue(const half_t *base, const unsigned (&off)[NLOAD], unsigned lds_wave)
+    __device__ static inline void issue(const half_t *base, long ld, unsigned voff, unsigned lds_wave)
     {
 #pragma unroll
-        for (int i = 0; i < NLOAD; i++) lds_dma16(base, off[i], lds_wave + (unsigned)(i * NT * 16));
+        for (int i = 0; i < NLOAD; i++) lds_dma16(base + load_delta(i, ld), voff, lds_wave + (unsigned)(i * NT * 16));
     }
 };
 
 // --------------------------------------------------------- fragment reads --
-// Lane byte offset (within the operand's LDS tile) of the fragment of MFMA
-// tile 0, k-step 0; tile t / k-step ks / half h add compile-time constants.
+// Lane byte offsets (within the operand's LDS slot) of the wavefront's
+// fragments; MFMA tile t and step-in-slot h add compile-time constants.
 template <int R, bool KMAJOR>
 struct frag_reader {
-    static constexpr int R16 = R / 16;
-    int base0, base1;  // K-major: one lane offset per k-step (the XOR involves ks)
+    static constexpr int READS_PER_FRAG = KMAJOR ? 1 : 2;
+    int base[4];  // K-major: [h] (the XOR involves h); I-major: [t % 4]
 
     __device__ inline void init(int wave_row0, int lane)
     {
         const int j = lane & 15, q = lane >> 4;
         if constexpr (KMAJOR) {
             const int r = wave_row0 + j;
-            base0 = (r * 8 + ((0 + q) ^ ((j >> 1) & 7))) * 16;
-            base1 = (r * 8 + ((4 + q) ^ ((j >> 1) & 7))) * 16;
+            base[0] = (r * 8 + ((0 + q) ^ ((j >> 1) & 7))) * 16;
+            base[1] = (r * 8 + ((4 + q) ^ ((j >> 1) & 7))) * 16;
+            base[2] = base[3] = 0;
         } else {
-            base0 = ((2 * (q >> 1)) * R16 + wave_row0 / 16) * 256 + (q & 1) * 128 + j * 8;
-            base1 = 0;
+            const int jq = j >> 2, jr = j & 3;
+            const int g = ((jq >> 1) & 1) | ((q & 1) << 1);  // i_major_swizzle of this lane's k
+            const int w16 = wave_row0 / 16;
+#pragma unroll
+            for (int m = 0; m < 4; m++)
+                base[m] = (w16 / 4) * 8192 + (8 * q + jq) * 128 + jr * 8 + ((((w16 & 3) + m) & 3) ^ g) * 32;
         }
     }
 
-    template <int T, int KS>
-    __device__ inline half8_t read(MIW_LDS const char *tile) const
+    template <int T, int H>
+    __device__ inline half8_t read(MIW_LDS const char *slot) const
     {
         if constexpr (KMAJOR) {
-            const int off = (KS == 0 ? base0 : base1) + T * 2048;
-            return *(MIW_LDS const half8_t *)(tile + off);
+            return *(MIW_LDS const half8_t *)(slot + base[H] + T * 2048);
         } else {
-            const int off = base0 + KS * (4 * R16 * 256) + T * 256;
-            fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(tile + off));
-            fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(tile + off + R16 * 256));
+            const int off = base[T & 3] + (T >> 2) * 8192 + H * 4096;
+            fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(slot + off));
+            fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(slot + off + 512));
             uint2_t l2 = __builtin_bit_cast(uint2_t, lo), h2 = __builtin_bit_cast(uint2_t, hi);
             uint4_t v = {l2[0], l2[1], h2[0], h2[1]};
             return __builtin_bit_cast(half8_t, v);
@@ -158,6 +190,28 @@ struct frag_reader {
 
 __device__ inline float round_through_half(float v) { return (float)(half_t)v; }
 
+// Scheduling hint for one pipeline step: the LDS reads of the next step's
+// fragments go first, one per MFMA, so that they are spread under matrix-core
+// work yet complete well before the step ends; the remaining MFMAs follow.
+template <int NREAD, int NMFMA, int I>
+__device__ inline void interleave_one()
+{
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+    if constexpr (I < NMFMA) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+}
+template <int NREAD, int NMFMA, int... I>
+__device__ inline void reads_first_then_mfma(std::integer_sequence<int, I...>)
+{
+    (interleave_one<NREAD, NMFMA, I>(), ...);
+    if constexpr (NMFMA > NREAD) __builtin_amdgcn_sched_group_barrier(0x008, NMFMA - NREAD, 0);
+}
+
+template <int TI, int TJ>
+struct frag_set {
+    half8_t x[TI];
+    half8_t y[TJ];
+};
+
 // ----------------------------------------------------------------- kernel --
 template <int BI, int BJ, int WI, int WJ, bool XK, bool YK, class CT, class DT, bool F16ACC>
 __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
@@ -165,9 +219,14 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
     constexpr int NT = WI * WJ * 64;
     constexpr int WTI = BI / WI, WTJ = BJ / WJ;
     constexpr int TI = WTI / 16, TJ = WTJ / 16;
-    constexpr int XBYTES = BI * BK * 2, YBYTES = BJ * BK * 2, STAGE = XBYTES + YBYTES;
-    using xload = tile_loader<BI, XK, NT>;
-    using yload = tile_loader<BJ, YK, NT>;
+    constexpr int XBYTES = BI * KGRAN * 2, YBYTES = BJ * KGRAN * 2, SLOT = XBYTES + YBYTES;
+    using xload = slot_loader<BI, XK, NT>;
+    using yload = slot_loader<BJ, YK, NT>;
+    using xreader = frag_reader<BI, XK>;
+    using yreader = frag_reader<BJ, YK>;
+    constexpr int NREAD = TI * xreader::READS_PER_FRAG + TJ * yreader::READS_PER_FRAG;
+    constexpr int NMFMA = TI * TJ;
+    static_assert(WTI % 32 == 0 && WTJ % 32 == 0, "wave tile");
 
     extern __shared__ __attribute__((aligned(128))) char smem[];
     MIW_LDS char *lds = (MIW_LDS char *)smem;
@@ -204,15 +263,13 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
 
     const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
     const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);
-    const long xstep = XK ? BK : (long)BK * p.ldx;
-    const long ystep = YK ? BK : (long)BK * p.ldy;
+    const long xstep = XK ? KGRAN : (long)KGRAN * p.ldx;
+    const long ystep = YK ? KGRAN : (long)KGRAN * p.ldy;
+    const unsigned xoff = xload::lane_offset(tid, (int)p.ldx);
+    const unsigned yoff = yload::lane_offset(tid, (int)p.ldy);
 
-    unsigned xoff[xload::NLOAD], yoff[yload::NLOAD];
-    xload::offsets(tid, (int)p.ldx, xoff);
-    yload::offsets(tid, (int)p.ldy, yoff);
-
-    frag_reader<BI, XK> xr;
-    frag_reader<BJ, YK> yr;
+    xreader xr;
+    yreader yr;
     xr.init(wi * WTI, lane);
     yr.init(wj * WTJ, lane);
 
@@ -245,11 +302,6 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
         return c;
     };
 
-    // First K-tile on its way before anything else.
-    const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
-    xload::issue(X, xoff, wave_dst);
-    yload::issue(Y, yoff, wave_dst + XBYTES);
-
     if constexpr (F16ACC) {
         // acc = half(beta * C): the Float16 accumulator starts as the C operand.
         if (p.use_c) {
@@ -265,42 +317,43 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
             };
             if (p.c_trans) init(true);
             else init(false);
+            // these were ordinary loads: drain them before the hand-counted ones start
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
     }
 
-    const int KT = p.K / BK;
-    for (int kt = 0; kt < KT; kt++) {
-        MIW_WAIT_VMCNT(0);
-        __syncthreads();
-        const int cur = (kt & 1) * STAGE;
-        if (kt + 1 < KT) {
-            X += xstep;
-            Y += ystep;
-            const int nxt = STAGE - cur;
-            xload::issue(X, xoff, wave_dst + nxt);
-            yload::issue(Y, yoff, wave_dst + nxt + XBYTES);
-        }
-        MIW_LDS const char *xt = lds + cur;
-        MIW_LDS const char *yt = lds + cur + XBYTES;
+    const int NP = p.K / KGRAN;  // slots' worth of K ("pairs" of steps)
+    const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
+    int next = 0;  // next pair to request
+    auto issue_next = [&]() {
+        const unsigned dst = wave_dst + (unsigned)((next & (NSLOT - 1)) * SLOT);
+        xload::issue(X, p.ldx, xoff, dst);
+        yload::issue(Y, p.ldy, yoff, dst + XBYTES);
+        X += xstep;
+        Y += ystep;
+        next++;
+    };
 
-        half8_t xf[2][TI], yf[2][TJ];
-        [&]<int... A>(__attribute__((unused)) std::integer_sequence<int, A...>) {
-            ((xf[0][A] = xr.template read<A, 0>(xt)), ...);
-            ((xf[1][A] = xr.template read<A, 1>(xt)), ...);
-        }(std::make_integer_sequence<int, TI>{});
-        [&]<int... B>(__attribute__((unused)) std::integer_sequence<int, B...>) {
-            ((yf[0][B] = yr.template read<B, 0>(yt)), ...);
-            ((yf[1][B] = yr.template read<B, 1>(yt)), ...);
-        }(std::make_integer_sequence<int, TJ>{});
+    auto read_frags = [&]<int H>(frag_set<TI, TJ> &f, int slot, std::integral_constant<int, H>) {
+        MIW_LDS const char *xs = lds + slot * SLOT;
+        MIW_LDS const char *ys = xs + XBYTES;
+        [&]<int... A>(std::integer_sequence<int, A...>) { ((f.x[A] = xr.template read<A, H>(xs)), ...); }
+        (std::make_integer_sequence<int, TI>{});
+        [&]<int... B>(std::integer_sequence<int, B...>) { ((f.y[B] = yr.template read<B, H>(ys)), ...); }
+        (std::make_integer_sequence<int, TJ>{});
+    };
+    constexpr std::integral_constant<int, 0> first_half{};
+    constexpr std::integral_constant<int, 1> second_half{};
 
+    auto multiply = [&](const frag_set<TI, TJ> &f) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++)
+        for (int a = 0; a < TI; a++)
 #pragma unroll
-            for (int a = 0; a < TI; a++)
-#pragma unroll
-                for (int b = 0; b < TJ; b++)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[ks][a], yf[ks][b], acc[a][b], 0, 0, 0);
-
+            for (int b = 0; b < TJ; b++)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.x[a], f.y[b], acc[a][b], 0, 0, 0);
+    };
+    auto hint = [&]() { reads_first_then_mfma<NREAD, NMFMA>(std::make_integer_sequence<int, NREAD>{}); };
+    auto round_acc = [&]() {
         if constexpr (F16ACC) {
 #pragma unroll
             for (int a = 0; a < TI; a++)
@@ -309,7 +362,41 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
 #pragma unroll
                     for (int v = 0; v < 4; v++) acc[a][b][v] = round_through_half(acc[a][b][v]);
         }
+    };
+
+    // Prologue: both slots requested, pair 0 published; step 0 runs while the
+    // second half of pair 0 is fetched into the other register set.
+    constexpr int LPAIR = xload::NLOAD + yload::NLOAD;  // loads per thread and pair
+    frag_set<TI, TJ> f0, f1;
+    issue_next();
+    if (NP > 1) {
+        issue_next();
+        wait_loads_and_barrier<LPAIR>();
+    } else {
+        wait_loads_and_barrier<0>();
     }
+    read_frags(f0, 0, first_half);
+    asm volatile("" ::: "memory");
+    read_frags(f1, 0, second_half);
+    multiply(f0);
+    hint();
+
+    // Pair p+1 is published at the top of the trip, pair p+2 requested into the
+    // slot pair p has just vacated; then steps 2p+1 and 2p+2.
+    for (int pr = 0; pr + 1 < NP; pr++) {
+        wait_loads_and_barrier<0>();
+        if (next < NP) issue_next();
+        const int slot = (pr + 1) & (NSLOT - 1);
+        read_frags(f0, slot, first_half);
+        multiply(f1);
+        hint();
+        round_acc();
+        read_frags(f1, slot, second_half);
+        multiply(f0);
+        hint();
+    }
+    multiply(f1);
+    round_acc();
 
     // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
     auto epilogue = [&](bool with_c, bool trans) {
@@ -345,17 +432,17 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
 
 static const tiled_variant g_variants[] = {
     // name                 bm   bn  bk  wm wn st  lds
-    {"tile256x256_w2x4", 256, 256, 64, 2, 4, 2, 2 * (256 + 256) * 128},
-    {"tile256x256_w4x2", 256, 256, 64, 4, 2, 2, 2 * (256 + 256) * 128},
-    {"tile256x128_w2x2", 256, 128, 64, 2, 2, 2, 2 * (256 + 128) * 128},
-    {"tile128x256_w2x2", 128, 256, 64, 2, 2, 2, 2 * (128 + 256) * 128},
-    {"tile128x128_w2x2", 128, 128, 64, 2, 2, 2, 2 * (128 + 128) * 128},
-    {"tile64x64_w2x2", 64, 64, 64, 2, 2, 2, 2 * (64 + 64) * 128},
+    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, NSLOT, NSLOT * (256 + 256) * KGRAN * 2},
+    {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, NSLOT, NSLOT * (256 + 256) * KGRAN * 2},
+    {"tile256x128_w2x2", 256, 128, KGRAN, 2, 2, NSLOT, NSLOT * (256 + 128) * KGRAN * 2},
+    {"tile128x256_w2x2", 128, 256, KGRAN, 2, 2, NSLOT, NSLOT * (128 + 256) * KGRAN * 2},
+    {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, NSLOT, NSLOT * (128 + 128) * KGRAN * 2},
+    {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, NSLOT, NSLOT * (64 + 64) * KGRAN * 2},
 };
 
 int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }
 const tiled_variant &tiled_variant_at(int i) { return g_variants[i]; }
-int tiled_f16acc_chunk() { return BK; }
+int tiled_f16acc_chunk() { return KGRAN; }
 
 template <int BI, int BJ, int WI, int WJ, class CT, class DT, bool F16ACC>
 static const void *pick_layout(bool xk, bool yk)
@@ -381,7 +468,7 @@ static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, 
 {
     switch (i) {
         case 0: return pick_types<256, 256, 2, 4>(xk, yk, c_type, d_type, f16acc);
-        case 1: return pick_types<256, 256, 4, 2>(xk, yk, c_type, d_type, f16acc);
+        case 1: return pick_types<256, 256, 2, 2>(xk, yk, c_type, d_type, f16acc);
         case 2: return pick_types<256, 128, 2, 2>(xk, yk, c_type, d_type, f16acc);
         case 3: return pick_types<128, 256, 2, 2>(xk, yk, c_type, d_type, f16acc);
         case 4: return pick_types<128, 128, 2, 2>(xk, yk, c_type, d_type, f16acc);
