@@ -164,6 +164,10 @@ int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc,
         if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk)) continue;
         const miw::tiled_variant &v = miw::tiled_variant_at(i);
         const long wgs = (I / v.bm) * (J / v.bn) * p.batch;
+        // A deep LDS ring on a small tile pays when one workgroup per CU runs a long K loop;
+        // with more workgroups than CUs the shallow ring lets two of them share a CU.
+        const bool deep_small = v.stages > 2 && v.bm * v.bn <= 128 * 128 && v.bm >= 128;
+        if (deep_small && (wgs > cus || p.K / v.bk < 2 * v.stages)) continue;
         if (wgs >= cus) return i + 1;
         if (wgs > best_wgs) { best = i; best_wgs = wgs; }
     }

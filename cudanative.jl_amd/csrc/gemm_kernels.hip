@@ -15,7 +15,7 @@
 // (A row-major / B column-major) and "I-major" otherwise; likewise Y.
 //
 // Pipeline.  K is consumed in steps of 32 k-values (one MFMA k-step), fetched
-// in pairs: LDS holds two slots of 64 k-values.  While the matrix cores work
+// in pairs: LDS holds two to four slots of 64 k-values (as many as fit).  While the matrix cores work
 // through the fragments of step s out of one register set, the fragments of
 // step s+1 are read from LDS into a second set (reads first, so that they have
 // landed long before the step ends), and the direct-to-LDS loads of the next
@@ -56,7 +56,6 @@ typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
 
 constexpr int BKS = 32;    // k-values per pipeline step (one MFMA k-step)
 constexpr int KGRAN = 64;  // k-values per LDS slot and K granularity of the kernel
-constexpr int NSLOT = 2;   // LDS slots
 
 struct tiled_params {
     const half_t *X;
@@ -190,22 +189,6 @@ struct frag_reader {
 
 __device__ inline float round_through_half(float v) { return (float)(half_t)v; }
 
-// Scheduling hint for one pipeline step: the LDS reads of the next step's
-// fragments go first, one per MFMA, so that they are spread under matrix-core
-// work yet complete well before the step ends; the remaining MFMAs follow.
-template <int NREAD, int NMFMA, int I>
-__device__ inline void interleave_one()
-{
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-    if constexpr (I < NMFMA) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-}
-template <int NREAD, int NMFMA, int... I>
-__device__ inline void reads_first_then_mfma(std::integer_sequence<int, I...>)
-{
-    (interleave_one<NREAD, NMFMA, I>(), ...);
-    if constexpr (NMFMA > NREAD) __builtin_amdgcn_sched_group_barrier(0x008, NMFMA - NREAD, 0);
-}
-
 template <int TI, int TJ>
 struct frag_set {
     half8_t x[TI];
@@ -213,8 +196,15 @@ struct frag_set {
 };
 
 // ----------------------------------------------------------------- kernel --
-template <int BI, int BJ, int WI, int WJ, bool XK, bool YK, class CT, class DT, bool F16ACC>
-__global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
+// Wavefronts per SIMD the register allocation aims at: two whenever the
+// accumulators (BI*BJ/NT floats per lane) leave room for the fragments in 256
+// registers, which also keeps them in ordinary VGPRs where the fp16-accumulate
+// rounding can reach them without copies.
+constexpr int waves_per_simd(int bi, int bj, int nt) { return bi * bj / nt <= 128 ? 2 : 1; }
+
+template <int BI, int BJ, int WI, int WJ, int NSLOT, bool XK, bool YK, class CT, class DT, bool F16ACC>
+__global__ __launch_bounds__(WI *WJ * 64) __attribute__((amdgpu_waves_per_eu(waves_per_simd(BI, BJ, WI *WJ * 64))))
+void k_gemm_tiled(tiled_params p)
 {
     constexpr int NT = WI * WJ * 64;
     constexpr int WTI = BI / WI, WTJ = BJ / WJ;
@@ -324,79 +314,123 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
 
     const int NP = p.K / KGRAN;  // slots' worth of K ("pairs" of steps)
     const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
-    int next = 0;  // next pair to request
-    auto issue_next = [&]() {
-        const unsigned dst = wave_dst + (unsigned)((next & (NSLOT - 1)) * SLOT);
-        xload::issue(X, p.ldx, xoff, dst);
-        yload::issue(Y, p.ldy, yoff, dst + XBYTES);
-        X += xstep;
-        Y += ystep;
+    constexpr int NLX = xload::NLOAD, NLY = yload::NLOAD, LPAIR = NLX + NLY;  // loads per thread and pair
+    int next = 0;          // next pair to request
+    int wslot = 0;         // the slot it goes to
+    unsigned dma_dst = 0;  // this wavefront's first destination byte in that slot
+    auto begin_request = [&]() { dma_dst = wave_dst + (unsigned)(wslot * SLOT); };
+    // Load number I of the pair being requested.
+    auto request_one = [&]<int I>(std::integral_constant<int, I>) {
+        if constexpr (I < NLX)
+            lds_dma16(X + xload::load_delta(I, p.ldx), xoff, dma_dst + (unsigned)(I * NT * 16));
+        else
+            lds_dma16(Y + yload::load_delta(I - NLX, p.ldy), yoff, dma_dst + XBYTES + (unsigned)((I - NLX) * NT * 16));
+    };
+    // Past the end of K the last pair is requested again, into a slot nobody
+    // reads any more: the pipeline stays free of branches.
+    auto end_request = [&]() {
         next++;
+        wslot = wslot + 1 == NSLOT ? 0 : wslot + 1;
+        const bool more = next < NP;
+        X += more ? xstep : 0;
+        Y += more ? ystep : 0;
+    };
+    auto request_pair = [&]() {
+        begin_request();
+        [&]<int... I>(std::integer_sequence<int, I...>) { (request_one(std::integral_constant<int, I>{}), ...); }
+        (std::make_integer_sequence<int, LPAIR>{});
+        end_request();
     };
 
-    auto read_frags = [&]<int H>(frag_set<TI, TJ> &f, int slot, std::integral_constant<int, H>) {
+    frag_set<TI, TJ> f0, f1;
+    // Fragment unit U of a step: the TI x-fragments, then the TJ y-fragments.
+    auto fetch_unit = [&]<int U, int H>(frag_set<TI, TJ> &f, MIW_LDS const char *xs, std::integral_constant<int, U>,
+                                        std::integral_constant<int, H>) {
+        if constexpr (U < TI) f.x[U] = xr.template read<U, H>(xs);
+        else f.y[U - TI] = yr.template read<U - TI, H>(xs + XBYTES);
+    };
+    constexpr int NUNIT = TI + TJ;
+    // One pipeline step, in source order and pinned there: before MFMA m the
+    // fragment unit m of the next step is fetched from LDS (all of them early
+    // in the step, so they have landed long before it ends); from MFMA
+    // NUNIT on, direct-to-LDS loads DMA_LO..DMA_HI-1 of the pair being
+    // requested are issued one per MFMA, in the shadow of the matrix cores.
+    // fp16 accumulate: the tile an MFMA of the pair's second step has just
+    // finished is rounded to Float16 two MFMAs later, in the shadow of the
+    // matrix cores, instead of all tiles at once after the step.
+    constexpr int ROUND_LAG = 2;
+    auto round_tile = [&](int m) {
+        const int a = m / TJ, b = m % TJ;
+        half4_t h = __builtin_convertvector(acc[a][b], half4_t);
+        acc[a][b] = __builtin_convertvector(h, float4_t);
+    };
+    auto step = [&]<int H, int DMA_LO, int DMA_HI>(const frag_set<TI, TJ> &cur, frag_set<TI, TJ> &nxt, int slot,
+                                                   std::integral_constant<int, H> h, std::integral_constant<int, DMA_LO>,
+                                                   std::integral_constant<int, DMA_HI>) {
+        constexpr bool ROUND = F16ACC && H == 0;  // the step that fetches a first half is the pair's second step
         MIW_LDS const char *xs = lds + slot * SLOT;
-        MIW_LDS const char *ys = xs + XBYTES;
-        [&]<int... A>(std::integer_sequence<int, A...>) { ((f.x[A] = xr.template read<A, H>(xs)), ...); }
-        (std::make_integer_sequence<int, TI>{});
-        [&]<int... B>(std::integer_sequence<int, B...>) { ((f.y[B] = yr.template read<B, H>(ys)), ...); }
-        (std::make_integer_sequence<int, TJ>{});
+        constexpr int NDMA = DMA_HI - DMA_LO;
+        // big steps: after the fragment reads; small steps are latency bound: at once
+        constexpr int DMA_FROM = (NMFMA >= 32 && NUNIT + NDMA <= NMFMA) ? NUNIT : 0;
+        [&]<int... Mi>(std::integer_sequence<int, Mi...>) {
+            (([&] {
+                 constexpr int m = Mi;
+                 if constexpr (m < NUNIT) fetch_unit(nxt, xs, std::integral_constant<int, m>{}, h);
+                 constexpr int a = m / TJ, b = m % TJ;
+                 acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.x[a], cur.y[b], acc[a][b], 0, 0, 0);
+                 if constexpr (m >= DMA_FROM && m - DMA_FROM < NDMA) {
+                     __builtin_amdgcn_sched_barrier(0);
+                     request_one(std::integral_constant<int, DMA_LO + (m - DMA_FROM)>{});
+                 }
+                 if constexpr (ROUND && m >= ROUND_LAG) round_tile(m - ROUND_LAG);
+                 __builtin_amdgcn_sched_barrier(0);
+             }()),
+             ...);
+        }(std::make_integer_sequence<int, NMFMA>{});
+        if constexpr (ROUND)
+#pragma unroll
+            for (int m = NMFMA > ROUND_LAG ? NMFMA - ROUND_LAG : 0; m < NMFMA; m++) round_tile(m);
+        // tiles with fewer MFMAs than fragment units or loads: the rest follows the last MFMA
+        if constexpr (NUNIT > NMFMA)
+            [&]<int... U>(std::integer_sequence<int, U...>) {
+                (fetch_unit(nxt, xs, std::integral_constant<int, NMFMA + U>{}, h), ...);
+            }(std::make_integer_sequence<int, NUNIT - NMFMA>{});
+        if constexpr (NDMA > NMFMA - DMA_FROM)
+            [&]<int... I>(std::integer_sequence<int, I...>) {
+                (request_one(std::integral_constant<int, DMA_LO + (NMFMA - DMA_FROM) + I>{}), ...);
+            }(std::make_integer_sequence<int, NDMA - (NMFMA - DMA_FROM)>{});
     };
     constexpr std::integral_constant<int, 0> first_half{};
     constexpr std::integral_constant<int, 1> second_half{};
+    constexpr std::integral_constant<int, 0> dma_begin{};
+    constexpr std::integral_constant<int, LPAIR / 2> dma_mid{};
+    constexpr std::integral_constant<int, LPAIR> dma_end{};
 
-    auto multiply = [&](const frag_set<TI, TJ> &f) {
+    // Prologue: every slot requested, pair 0 published and its first fragments fetched.
 #pragma unroll
-        for (int a = 0; a < TI; a++)
-#pragma unroll
-            for (int b = 0; b < TJ; b++)
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.x[a], f.y[b], acc[a][b], 0, 0, 0);
-    };
-    auto hint = [&]() { reads_first_then_mfma<NREAD, NMFMA>(std::make_integer_sequence<int, NREAD>{}); };
-    auto round_acc = [&]() {
-        if constexpr (F16ACC) {
-#pragma unroll
-            for (int a = 0; a < TI; a++)
-#pragma unroll
-                for (int b = 0; b < TJ; b++)
-#pragma unroll
-                    for (int v = 0; v < 4; v++) acc[a][b][v] = round_through_half(acc[a][b][v]);
-        }
-    };
+    for (int s = 0; s < NSLOT; s++) request_pair();
+    wait_loads_and_barrier<(NSLOT - 1) * LPAIR>();
+    [&]<int... U>(std::integer_sequence<int, U...>) {
+        (fetch_unit(f0, lds, std::integral_constant<int, U>{}, first_half), ...);
+    }(std::make_integer_sequence<int, NUNIT>{});
 
-    // Prologue: both slots requested, pair 0 published; step 0 runs while the
-    // second half of pair 0 is fetched into the other register set.
-    constexpr int LPAIR = xload::NLOAD + yload::NLOAD;  // loads per thread and pair
-    frag_set<TI, TJ> f0, f1;
-    issue_next();
-    if (NP > 1) {
-        issue_next();
-        wait_loads_and_barrier<LPAIR>();
-    } else {
-        wait_loads_and_barrier<0>();
+    // Trip pr: step 2pr (second half of pair pr's slot is fetched; nothing to
+    // request yet: the slot is still being read), barrier (pair pr+1 has
+    // landed, pair pr's slot is free), step 2pr+1 (first half of pair pr+1 is
+    // fetched while pair pr+NSLOT is requested into the freed slot; NSLOT-2
+    // younger pairs stay in flight across the barrier).  On the last trip
+    // nothing new lands; its odd step reads another slot's stale bytes into
+    // registers nobody uses.
+    int rslot = 0;
+    for (int pr = 0; pr < NP; pr++) {
+        step(f0, f1, rslot, second_half, dma_begin, dma_begin);
+        wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
+        rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
+        begin_request();
+        step(f1, f0, rslot, first_half, dma_begin, dma_end);
+        end_request();
     }
-    read_frags(f0, 0, first_half);
-    asm volatile("" ::: "memory");
-    read_frags(f1, 0, second_half);
-    multiply(f0);
-    hint();
-
-    // Pair p+1 is published at the top of the trip, pair p+2 requested into the
-    // slot pair p has just vacated; then steps 2p+1 and 2p+2.
-    for (int pr = 0; pr + 1 < NP; pr++) {
-        wait_loads_and_barrier<0>();
-        if (next < NP) issue_next();
-        const int slot = (pr + 1) & (NSLOT - 1);
-        read_frags(f0, slot, first_half);
-        multiply(f1);
-        hint();
-        round_acc();
-        read_frags(f1, slot, second_half);
-        multiply(f0);
-        hint();
-    }
-    multiply(f1);
-    round_acc();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may outlive the workgroup's LDS
 
     // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
     auto epilogue = [&](bool with_c, bool trans) {
@@ -431,48 +465,50 @@ __global__ __launch_bounds__(WI *WJ * 64) void k_gemm_tiled(tiled_params p)
 // --------------------------------------------------------------- variants --
 
 static const tiled_variant g_variants[] = {
-    // name                 bm   bn  bk  wm wn st  lds
-    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, NSLOT, NSLOT * (256 + 256) * KGRAN * 2},
-    {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, NSLOT, NSLOT * (256 + 256) * KGRAN * 2},
-    {"tile256x128_w2x2", 256, 128, KGRAN, 2, 2, NSLOT, NSLOT * (256 + 128) * KGRAN * 2},
-    {"tile128x256_w2x2", 128, 256, KGRAN, 2, 2, NSLOT, NSLOT * (128 + 256) * KGRAN * 2},
-    {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, NSLOT, NSLOT * (128 + 128) * KGRAN * 2},
-    {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, NSLOT, NSLOT * (64 + 64) * KGRAN * 2},
+    // name                    bm   bn  bk     wm wn slots lds
+    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2},
+    {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2},
+    {"tile256x128_w2x2", 256, 128, KGRAN, 2, 2, 3, 3 * (256 + 128) * KGRAN * 2},
+    {"tile128x256_w2x2", 128, 256, KGRAN, 2, 2, 3, 3 * (128 + 256) * KGRAN * 2},
+    {"tile128x128_w2x2_s4", 128, 128, KGRAN, 2, 2, 4, 4 * (128 + 128) * KGRAN * 2},
+    {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2},
+    {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, 4, 4 * (64 + 64) * KGRAN * 2},
 };
 
 int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }
 const tiled_variant &tiled_variant_at(int i) { return g_variants[i]; }
 int tiled_f16acc_chunk() { return KGRAN; }
 
-template <int BI, int BJ, int WI, int WJ, class CT, class DT, bool F16ACC>
+template <int BI, int BJ, int WI, int WJ, int NS, class CT, class DT, bool F16ACC>
 static const void *pick_layout(bool xk, bool yk)
 {
-    if (xk && yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, true, true, CT, DT, F16ACC>;
-    if (xk && !yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, true, false, CT, DT, F16ACC>;
-    if (!xk && yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, false, true, CT, DT, F16ACC>;
-    return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, false, false, CT, DT, F16ACC>;
+    if (xk && yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, NS, true, true, CT, DT, F16ACC>;
+    if (xk && !yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, NS, true, false, CT, DT, F16ACC>;
+    if (!xk && yk) return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, NS, false, true, CT, DT, F16ACC>;
+    return (const void *)k_gemm_tiled<BI, BJ, WI, WJ, NS, false, false, CT, DT, F16ACC>;
 }
 
-template <int BI, int BJ, int WI, int WJ>
+template <int BI, int BJ, int WI, int WJ, int NS>
 static const void *pick_types(bool xk, bool yk, int c_type, int d_type, bool f16acc)
 {
-    if (f16acc) return pick_layout<BI, BJ, WI, WJ, half_t, half_t, true>(xk, yk);
-    if (c_type == 0 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, half_t, half_t, false>(xk, yk);
-    if (c_type == 0 && d_type == 1) return pick_layout<BI, BJ, WI, WJ, half_t, float, false>(xk, yk);
-    if (c_type == 1 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, float, half_t, false>(xk, yk);
-    return pick_layout<BI, BJ, WI, WJ, float, float, false>(xk, yk);
+    if (f16acc) return pick_layout<BI, BJ, WI, WJ, NS, half_t, half_t, true>(xk, yk);
+    if (c_type == 0 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, NS, half_t, half_t, false>(xk, yk);
+    if (c_type == 0 && d_type == 1) return pick_layout<BI, BJ, WI, WJ, NS, half_t, float, false>(xk, yk);
+    if (c_type == 1 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, NS, float, half_t, false>(xk, yk);
+    return pick_layout<BI, BJ, WI, WJ, NS, float, float, false>(xk, yk);
 }
 
 // Tile shape in canonical (I, J) terms: bm applies to I, bn to J.
 static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, bool f16acc)
 {
     switch (i) {
-        case 0: return pick_types<256, 256, 2, 4>(xk, yk, c_type, d_type, f16acc);
-        case 1: return pick_types<256, 256, 2, 2>(xk, yk, c_type, d_type, f16acc);
-        case 2: return pick_types<256, 128, 2, 2>(xk, yk, c_type, d_type, f16acc);
-        case 3: return pick_types<128, 256, 2, 2>(xk, yk, c_type, d_type, f16acc);
-        case 4: return pick_types<128, 128, 2, 2>(xk, yk, c_type, d_type, f16acc);
-        case 5: return pick_types<64, 64, 2, 2>(xk, yk, c_type, d_type, f16acc);
+        case 0: return pick_types<256, 256, 2, 4, 2>(xk, yk, c_type, d_type, f16acc);
+        case 1: return pick_types<256, 256, 2, 2, 2>(xk, yk, c_type, d_type, f16acc);
+        case 2: return pick_types<256, 128, 2, 2, 3>(xk, yk, c_type, d_type, f16acc);
+        case 3: return pick_types<128, 256, 2, 2, 3>(xk, yk, c_type, d_type, f16acc);
+        case 4: return pick_types<128, 128, 2, 2, 4>(xk, yk, c_type, d_type, f16acc);
+        case 5: return pick_types<128, 128, 2, 2, 2>(xk, yk, c_type, d_type, f16acc);
+        case 6: return pick_types<64, 64, 2, 2, 4>(xk, yk, c_type, d_type, f16acc);
     }
     return nullptr;
 }

@@ -195,7 +195,10 @@ def test_variant_table_and_selection(miw):
     by = {v["name"]: v["id"] for v in vs}
     # 4096^3 fills 256 CUs with 256x256 tiles; small or odd shapes fall to smaller tiles / fragment ops
     assert G.pick_variant(G.make_desc(4096, 4096, 4096)) == 1
-    assert vs[G.pick_variant(G.make_desc(128, 128, 128, batch=512)) - 1]["block"][:2] == (128, 128)
+    batched = vs[G.pick_variant(G.make_desc(128, 128, 128, batch=512)) - 1]
+    assert batched["block"][:2] == (128, 128) and batched["stages"] == 2      # two workgroups per CU
+    deep = vs[G.pick_variant(G.make_desc(2048, 2048, 2048)) - 1]
+    assert deep["block"][:2] == (128, 128) and deep["stages"] == 4            # one workgroup per CU, long K
     assert G.pick_variant(G.make_desc(48, 48, 48)) == by["fragment_ops"]
     assert G.pick_variant(G.make_desc(64, 64, 80)) == by["fragment_ops"]
     d = G.make_desc(2048, 2048, 2048, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
