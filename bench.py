@@ -4,7 +4,8 @@ baseline timed on this host).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--variant V] [--no-cpu]
 
-A step is one GEMM launch on inputs already resident in HBM.  `value` comes from the wall clock
+A step is one GEMM launch on inputs already resident in HBM.  Before the warm-up steps the same
+launch is repeated untimed for --spinup-seconds so that the clocks have left their idle state.  `value` comes from the wall clock
 around K back-to-back launches (synchronised on both sides); `roofline.achieved` from the HIP-event
 time over the same K launches, recorded on the launch stream, divided by K.
 """
@@ -25,8 +26,10 @@ PEAK_HBM_GBS = 8000.0
 # each scaled by what the counter reads for the library's copy kernel on 256 MiB; the summaries
 # and commands are under profiles/.  Configurations without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    "c2": int((257.3 + 73.0) * 2 ** 20),   # profiles/gemm_tiled_256x256_c2_4096cubed.md
-    "c5": int((64.1 + 32.0) * 2 ** 20),    # profiles/gemm_tiled_128x128_c5_batched128.md
+    "c2": int((256.1 + 69.5) * 2 ** 20),   # profiles/gemm_tiled_256x256_4096cubed_f32acc.md
+    "c3": int((56.1 + 8.0) * 2 ** 20),     # profiles/gemm_tiled_128x128_2048cubed_f16acc.md
+    "c4": int((160.1 + 33.6) * 2 ** 20),   # profiles/gemm_tiled_256x128_8192x1024x4096_mixed_layout.md
+    "c5": int((64.1 + 32.0) * 2 ** 20),    # profiles/gemm_tiled_128x128_batched_512x128cubed.md
 }
 
 CONFIGS = {
@@ -81,8 +84,11 @@ def cpu_baseline(orc, M, N, K, batch, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--spinup-seconds", type=float, default=0.3,
+                    help="untimed launches before the warm-up steps, until the GPU's power management has "
+                         "raised the clocks from idle (the first ~250 launches after idle run up to 20 %% slower)")
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
@@ -139,6 +145,11 @@ def main():
     ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
     m._lib.check(lib.miw_event_create(ctypes.byref(ev0)))
     m._lib.check(lib.miw_event_create(ctypes.byref(ev1)))
+    t_spin = time.perf_counter()
+    while time.perf_counter() - t_spin < args.spinup_seconds:
+        for _ in range(50):
+            G.gemm(dA, dB, dC, dD, desc)
+        m.synchronize()
     for _ in range(args.warmup):
         G.gemm(dA, dB, dC, dD, desc)
     m.synchronize()

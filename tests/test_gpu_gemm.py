@@ -79,6 +79,23 @@ def test_every_variant_exact_on_integer_inputs(gpu, orc, al, bl, dl):
         assert np.array_equal(D, orc.gemm(g, A, B, C)), (v["name"], al, bl, dl)
 
 
+@pytest.mark.parametrize("K", [64, 128, 320])
+def test_short_k_every_variant(gpu, orc, K):
+    """K of one, two and five LDS slots' worth: fewer slots' worth of K than the ring has slots,
+    and an odd count; bit-exact on integer inputs, against float64 on random ones."""
+    for v in _variants(gpu):
+        if v["fragment_ops"]:
+            continue
+        bm, bn = v["block"][:2]
+        g = orc.GemmDesc(M=bm, N=2 * bn, K=K, a_layout=orc.ROW, b_layout=orc.ROW)
+        A, B, C = _inputs(orc, g, 300 + v["id"], ints=True)
+        assert np.array_equal(_run(gpu, orc, g, A, B, C, variant=v["id"]), orc.gemm(g, A, B, C)), (v["name"], K)
+        g = orc.GemmDesc(M=2 * bm, N=bn, K=K)
+        A, B, C = _inputs(orc, g, 400 + v["id"])
+        D = _run(gpu, orc, g, A, B, C, variant=v["id"])
+        assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32, (v["name"], K)
+
+
 def test_identity_and_ones(gpu, orc):
     g = orc.GemmDesc(M=256, N=256, K=256)
     _, B, C = _inputs(orc, g, 3)
