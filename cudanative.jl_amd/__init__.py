@@ -13,6 +13,7 @@ from .array import AS, DeviceArray, DevicePtr, CU_NULL, pointer
 from .execution import HostKernel, Stream, cuda, cufunction, cudaconvert, kernel_names, synchronize
 from . import wmma as WMMA
 from . import gemm as GEMM
+from . import reflection
 
 CuHostArray = DeviceArray
 

@@ -80,6 +80,7 @@ class GemmVariantInfo(ctypes.Structure):
         ("block_m", ctypes.c_int), ("block_n", ctypes.c_int), ("block_k", ctypes.c_int),
         ("waves_m", ctypes.c_int), ("waves_n", ctypes.c_int),
         ("stages", ctypes.c_int), ("lds_bytes", ctypes.c_int), ("fragment_ops", ctypes.c_int),
+        ("f16_accumulate", ctypes.c_int),
     ]
 
 

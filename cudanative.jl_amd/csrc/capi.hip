@@ -147,7 +147,9 @@ bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f
     if (p.use_c && (p.ldc % cper || p.sc % cper)) return false;
     // 32-bit offsets inside one operand tile
     if (p.lda * 256 >= (1l << 31) || p.ldb * 256 >= (1l << 31)) return false;
-    if (f16acc && (p.alpha != 1.0f || (acc_chunk != 0 && acc_chunk != miw::tiled_f16acc_chunk()))) return false;
+    if (f16acc && (!miw::tiled_supports_f16acc(i) || p.alpha != 1.0f ||
+                   (acc_chunk != 0 && acc_chunk != miw::tiled_f16acc_chunk())))
+        return false;
     return true;
 }
 
@@ -193,7 +195,7 @@ int run_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, hip
                     "gemm: variant %d (%s) needs tile-divisible sizes, 16-byte aligned operands and leading "
                     "dimensions%s",
                     variant, miw::tiled_variant_at(variant - 1).name,
-                    f16acc ? ", alpha == 1 and its own acc_chunk" : "");
+                    f16acc ? ", alpha == 1, its own acc_chunk, and accumulators that fit in VGPRs" : "");
     HIP_TRY(miw::launch_gemm_tiled(variant - 1, p, d->c_type, d->d_type, f16acc, s));
     return 0;
 }
@@ -466,12 +468,14 @@ int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out)
         snprintf(out->name, sizeof(out->name), "fragment_ops");
         out->block_m = 16; out->block_n = 16; out->block_k = 16;
         out->waves_m = 1; out->waves_n = 1; out->stages = 1; out->lds_bytes = 0; out->fragment_ops = 1;
+        out->f16_accumulate = 1;
         return 0;
     }
     const miw::tiled_variant &v = miw::tiled_variant_at(variant - 1);
     snprintf(out->name, sizeof(out->name), "%s", v.name);
     out->block_m = v.bm; out->block_n = v.bn; out->block_k = v.bk;
     out->waves_m = v.wm; out->waves_n = v.wn; out->stages = v.stages; out->lds_bytes = v.lds_bytes;
+    out->f16_accumulate = miw::tiled_supports_f16acc(variant - 1) ? 1 : 0;
     return 0;
 }
 

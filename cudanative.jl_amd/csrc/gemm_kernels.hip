@@ -478,6 +478,11 @@ static const tiled_variant g_variants[] = {
 int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }
 const tiled_variant &tiled_variant_at(int i) { return g_variants[i]; }
 int tiled_f16acc_chunk() { return KGRAN; }
+bool tiled_supports_f16acc(int i)
+{
+    const tiled_variant &v = g_variants[i];
+    return waves_per_simd(v.bm, v.bn, v.wm * v.wn * 64) >= 2;
+}
 
 template <int BI, int BJ, int WI, int WJ, int NS, class CT, class DT, bool F16ACC>
 static const void *pick_layout(bool xk, bool yk)
@@ -491,7 +496,11 @@ static const void *pick_layout(bool xk, bool yk)
 template <int BI, int BJ, int WI, int WJ, int NS>
 static const void *pick_types(bool xk, bool yk, int c_type, int d_type, bool f16acc)
 {
-    if (f16acc) return pick_layout<BI, BJ, WI, WJ, NS, half_t, half_t, true>(xk, yk);
+    if (f16acc) {
+        // the rounding runs on the VALU: it needs the accumulators in ordinary VGPRs
+        if constexpr (waves_per_simd(BI, BJ, WI * WJ * 64) < 2) return nullptr;
+        else return pick_layout<BI, BJ, WI, WJ, NS, half_t, half_t, true>(xk, yk);
+    }
     if (c_type == 0 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, NS, half_t, half_t, false>(xk, yk);
     if (c_type == 0 && d_type == 1) return pick_layout<BI, BJ, WI, WJ, NS, half_t, float, false>(xk, yk);
     if (c_type == 1 && d_type == 0) return pick_layout<BI, BJ, WI, WJ, NS, float, half_t, false>(xk, yk);

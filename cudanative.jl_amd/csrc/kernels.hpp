@@ -47,6 +47,8 @@ int tiled_variant_count();
 const tiled_variant &tiled_variant_at(int i);
 // acc_chunk the tiled fp16-accumulate kernels round at.
 int tiled_f16acc_chunk();
+// Variants whose accumulators do not fit in ordinary VGPRs have no fp16-accumulate form.
+bool tiled_supports_f16acc(int i);
 // Launches tiled variant i.  The caller has checked divisibility by the tile,
 // 16-byte alignment of pointers and leading dimensions, and (for fp16
 // accumulate) alpha == 1 and c_type == d_type == Float16.

@@ -194,6 +194,7 @@ typedef struct miw_gemm_variant_info {
     int stages;
     int lds_bytes;
     int fragment_ops;   /* 1: built from load_a/load_b/mma on global memory, no LDS */
+    int f16_accumulate; /* 1: has a Float16-accumulate form (accumulators fit in ordinary VGPRs) */
 } miw_gemm_variant_info;
 int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
 /* Variant miw_gemm would pick for this descriptor. */

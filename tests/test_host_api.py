@@ -139,7 +139,7 @@ def test_struct_sizes_match_header(miw):
     L = miw._lib
     assert ctypes.sizeof(L.MacDesc) == 13 * 4 + 4 + 4 * 8      # 13 ints/floats, pad, 4 int64
     assert ctypes.sizeof(L.GemmDesc) == 7 * 8 + 11 * 4 + 4 + 5 * 8 + 8
-    assert ctypes.sizeof(L.GemmVariantInfo) == 64 + 8 * 4
+    assert ctypes.sizeof(L.GemmVariantInfo) == 64 + 9 * 4
     assert ctypes.sizeof(L.DeviceInfo) == 128 + 64 + 7 * 4 + 4 + 2 * 8 + 8
 
 
@@ -205,6 +205,13 @@ def test_variant_table_and_selection(miw):
     assert G.acc_chunk(d) == 64
     d = G.make_desc(48, 48, 48, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
     assert G.acc_chunk(d) == 16
+    # fp16 accumulate rounds on the VALU: offered only where a lane's accumulators fit in 128 VGPRs
+    for v in vs[:-1]:
+        per_lane = v["block"][0] * v["block"][1] // (v["waves"][0] * v["waves"][1] * 64)
+        assert v["f16_accumulate"] == (per_lane <= 128), v["name"]
+    assert vs[-1]["f16_accumulate"]
+    d = G.make_desc(4096, 4096, 4096, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
+    assert vs[G.pick_variant(d) - 1]["f16_accumulate"]
     names = miw.kernel_names()
     assert "wmma_mac_f32_f32" in names and "gemm_tile256x256_w2x4" in names
 

@@ -1,0 +1,63 @@
+"""Codegen checks on the compiled kernels (no GPU needed): the analogue of the reference's PTX
+string matches, test/device/wmma.jl:254-291 (store_d on a Global / Shared pointer must emit the
+.global. / .shared. instruction variants, not generic ones), plus resource usage of the GEMM."""
+import collections
+import re
+
+
+def _ops(text):
+    return collections.Counter(l.split()[0] for l in text.splitlines()
+                               if l.strip() and not l.strip().startswith(("<", ";")))
+
+
+def test_store_d_addressing(miw):
+    for T in ("float", "_Float16"):
+        isa = miw.reflection.code_gcn(f"k_frag_store<{T}>")
+        assert len(isa) == 1
+        ops = _ops(next(iter(isa.values())))
+        assert any(o.startswith("ds_write") for o in ops)          # LDS pointer overload -> ds_write
+        assert any(o.startswith("global_store") for o in ops)      # global pointer -> global_store
+        assert not any(o.startswith(("flat_store", "scratch_")) for o in ops)
+
+
+def test_load_addressing(miw):
+    for T in ("float", "_Float16"):
+        isa = miw.reflection.code_gcn(f"k_frag_load<{T}>")
+        assert len(isa) == 1
+        ops = _ops(next(iter(isa.values())))
+        assert any(o.startswith("ds_read") for o in ops) and any(o.startswith("global_load") for o in ops)
+        assert not any(o.startswith(("flat_load", "scratch_")) for o in ops)
+
+
+def test_fragment_mma_uses_the_16x16x16_matrix_instruction(miw):
+    isa = miw.reflection.code_gcn("k_frag_mma<float, float>")
+    assert _ops(next(iter(isa.values())))["v_mfma_f32_16x16x16_f16"] == 1
+
+
+def test_default_gemm_kernel_codegen_and_resources(miw):
+    name = "k_gemm_tiled<256, 256, 2, 4, 2, false, true, float, float, false>"    # column-major A and B, 8 waves
+    isa = miw.reflection.code_gcn(name)
+    assert len(isa) == 1
+    ops = _ops(next(iter(isa.values())))
+    assert ops["v_mfma_f32_16x16x32_f16"] >= 64                  # two unrolled steps of 8 x 4 tiles
+    assert ops["global_load_lds_dwordx4"] >= 8                   # direct-to-LDS operand loads
+    assert ops["ds_read_b64_tr_b16"] >= 32 and ops["ds_read_b128"] >= 8   # transpose reads for A, b128 for B
+    assert not any(o.startswith(("scratch_", "flat_", "ds_write", "v_accvgpr")) for o in ops)
+    res = {k: v for k, v in miw.reflection.kernel_resources().items() if name in k}
+    (r,) = res.values()
+    assert r["spills"] == 0 and r["scratch"] == 0 and r["max_threads"] == 512
+    assert r["vgpr"] + r["agpr"] <= 256                          # two wavefronts per SIMD
+    # both operands K-major: no transpose read at all
+    kk = miw.reflection.code_gcn("k_gemm_tiled<256, 256, 2, 4, 2, true, true, float, float, false>")
+    assert "ds_read_b64_tr_b16" not in _ops(next(iter(kk.values())))
+
+
+def test_no_tiled_kernel_spills_in_its_k_loop(miw):
+    # spills, where the allocator needs them at all, stay out of the loop that holds the MFMAs
+    for name, text in miw.reflection.code_gcn("k_gemm_tiled<").items():
+        lines = text.splitlines()
+        mfma = [i for i, l in enumerate(lines) if "v_mfma" in l]
+        assert mfma, name
+        # the K loop is the span between the first backward branch target and that branch
+        scratch_in_hot = [l for l in lines[mfma[0]:mfma[-1]] if re.match(r"\s*scratch_", l)]
+        assert len(scratch_in_hot) <= 8, (name, len(scratch_in_hot))
