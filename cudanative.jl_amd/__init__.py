@@ -14,6 +14,7 @@ from .execution import HostKernel, Stream, cuda, cufunction, cudaconvert, kernel
 from . import wmma as WMMA
 from . import gemm as GEMM
 from . import reflection
+from . import launch_overhead
 
 CuHostArray = DeviceArray
 

@@ -11,6 +11,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <ctime>
 #include <string>
 #include <vector>
 
@@ -533,6 +534,35 @@ int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, cons
     for (auto &e : ev) (void)hipEventDestroy(e);
     if (rc) return rc;
     if (he != hipSuccess) return hip_fail(he, "gemm_bench");
+    return 0;
+}
+
+int miw_launch_overhead_probe(int iters, int threads, float *cpu_us, float *gpu_us)
+{
+    if (!cpu_us || !gpu_us || iters < 1 || threads < 1 || threads > 1024)
+        return fail(MIW_ERR_INVALID_VALUE, "launch_overhead_probe: bad arguments");
+    float *buf = nullptr;
+    HIP_TRY(hipMalloc((void **)&buf, 4));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t he = hipEventCreate(&e0);
+    if (he == hipSuccess) he = hipEventCreate(&e1);
+    for (int i = 0; i < iters && he == hipSuccess; ++i) {
+        timespec t0, t1;
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        he = hipEventRecord(e0, nullptr);
+        if (he == hipSuccess) he = miw::launch_dummy_store(buf, threads, nullptr);
+        if (he == hipSuccess) he = hipEventRecord(e1, nullptr);
+        if (he == hipSuccess) he = hipEventSynchronize(e1);
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        float ms = 0.f;
+        if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+        cpu_us[i] = (float)((t1.tv_sec - t0.tv_sec) * 1e6 + (t1.tv_nsec - t0.tv_nsec) * 1e-3);
+        gpu_us[i] = ms * 1e3f;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(buf);
+    if (he != hipSuccess) return hip_fail(he, "launch_overhead_probe");
     return 0;
 }
 

@@ -381,6 +381,16 @@ hipError_t launch_gemm_fragops(const gemm_params &p, int c_type, int d_type, boo
     return hipGetLastError();
 }
 
+// The dummy kernel of the launch-overhead benchmark (test/perf/launch_overhead/cudanative.jl:9-12):
+// every lane of workgroup b stores 0 to ptr[b].
+__global__ void k_dummy_store(float *ptr) { ptr[blockIdx.x] = 0.f; }
+
+hipError_t launch_dummy_store(float *ptr, int threads, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_dummy_store, dim3(1), dim3(threads), 0, s, ptr);
+    return hipGetLastError();
+}
+
 // Host stubs exported to the named-kernel registry.
 const void *frag_kernel_symbol(const char *name)
 {
@@ -400,21 +410,22 @@ const void *frag_kernel_symbol(const char *name)
         {"frag_mma_f32_f32", (const void *)k_frag_mma<float, float>},
         {"wmma_mac_f32_f32", (const void *)k_wmma_mac<float, float>},
         {"gemm_fragops_f32_f32", (const void *)k_gemm_fragops<float, float, false>},
+        {"dummy_store", (const void *)k_dummy_store},
     };
     for (const auto &e : table)
         if (!__builtin_strcmp(e.n, name)) return e.f;
     return nullptr;
 }
 
-int frag_kernel_count() { return 14; }
+int frag_kernel_count() { return 15; }
 
 const char *frag_kernel_name(int i)
 {
     static const char *names[] = {"frag_load_f16",    "frag_load_f32",    "frag_store_f16",   "frag_store_f32",
                                   "frag_fill_f16",    "frag_fill_f32",    "frag_map_f16",     "frag_map_f32",
                                   "frag_mma_f16_f16", "frag_mma_f16_f32", "frag_mma_f32_f16", "frag_mma_f32_f32",
-                                  "wmma_mac_f32_f32", "gemm_fragops_f32_f32"};
-    return (i >= 0 && i < 14) ? names[i] : nullptr;
+                                  "wmma_mac_f32_f32", "gemm_fragops_f32_f32", "dummy_store"};
+    return (i >= 0 && i < 15) ? names[i] : nullptr;
 }
 
 }  // namespace miw

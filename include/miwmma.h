@@ -211,6 +211,13 @@ int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, cons
    of examples/peakflops.jl): measured TFLOP/s of the matrix cores alone. */
 int miw_mfma_peak_probe(int iters, double *tflops, void *stream);
 
+/* The raw-driver leg of the launch-overhead benchmark (test/perf/launch_overhead/cuda.c:60-80):
+   iters times { record event; launch the dummy kernel with `threads` lanes; record event;
+   synchronize }, all inside the library with no foreign-function hop; cpu_us[i] receives the
+   host wall time of iteration i and gpu_us[i] the time between the two events, both in
+   microseconds.  The other leg launches "dummy_store" through miw_launch from the host language. */
+int miw_launch_overhead_probe(int iters, int threads, float *cpu_us, float *gpu_us);
+
 /* Plain device copy kernel (16 B per lane), used to calibrate HBM counters. */
 int miw_copy_probe(void *dst, const void *src, size_t bytes, void *stream);
 

@@ -435,3 +435,20 @@ def test_device_array_semantics(gpu):
     assert gpu.pointer(d, 2).addr == d.ptr + 4 and gpu.pointer(d).addrspace == gpu.AS.Global
     info = gpu.device_info()
     assert info["arch"].startswith("gfx950") and info["wave_size"] == 64 and info["cu_count"] > 0
+
+
+# ---- test/perf/launch_overhead -----------------------------------------------------
+
+@pytest.mark.gpu
+def test_launch_overhead_benchmark_runs(gpu):
+    """The dummy kernel stores its zero; both legs report finite, positive, sub-millisecond means."""
+    buf = gpu.DeviceArray(np.full(8, 7.0, dtype=np.float32))
+    gpu.cuda("dummy_store", buf, threads=1000, blocks=3)
+    gpu.synchronize()
+    assert np.array_equal(buf.to_host(), np.array([0, 0, 0, 7, 7, 7, 7, 7], dtype=np.float32))
+    res = gpu.launch_overhead.run(gpu)
+    for leg in ("library", "host_language"):
+        for key in ("cpu_us", "gpu_us"):
+            mean, std = res[leg][key]
+            assert 0.0 < mean < 1000.0 and std >= 0.0, (leg, key, mean, std)
+    assert res["host_language"]["cpu_us"][0] >= 0.5 * res["library"]["cpu_us"][0]
