@@ -97,6 +97,19 @@ __device__ inline void lds_dma16(const void *base, unsigned voff, unsigned lds_a
                  : "memory", "m0");
 }
 
+// The same with a compile-time byte offset added to the global address.  The
+// instruction's offset field advances the LDS address as well as the global
+// one, so M0 is set back by as much.
+template <int IMM>
+__device__ inline void lds_dma16_imm(const void *base, unsigned voff, unsigned lds_addr)
+{
+    static_assert(IMM >= 0 && IMM < 4096, "instruction offset field");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+                 :
+                 : "s"(lds_addr - (unsigned)IMM), "v"(voff), "s"(base), "n"(IMM)
+                 : "memory", "m0");
+}
+
 __device__ inline int i_major_swizzle(int k) { return ((k >> 1) & 1) | (((k >> 3) & 1) << 1); }
 
 // ------------------------------------------------------------ slot loader --
@@ -201,6 +214,20 @@ struct frag_set {
 // registers, which also keeps them in ordinary VGPRs where the fp16-accumulate
 // rounding can reach them without copies.
 constexpr int waves_per_simd(int bi, int bj, int nt) { return bi * bj / nt <= 128 ? 2 : 1; }
+
+// MFMA tiles of C that one trip of the loop's tail folds into the accumulators
+// (0: the variant does not fold).  Folding needs the accumulators in ordinary
+// VGPRs, at most one pair in flight across a barrier, and LDS room for two
+// staging buffers of that many 1 KiB tiles per wavefront.  Only the 8-wavefront
+// tile folds: the 4-wavefront kernels issue half as many loads per thread again
+// and the register allocator answers the unrolled tail with spills.
+constexpr int fold_tiles(int bi, int bj, int nt, int nslot)
+{
+    if (waves_per_simd(bi, bj, nt) < 2 || nslot > 3 || nt != 512) return 0;
+    const int cpt = 2;
+    return nslot * (bi + bj) * KGRAN * 2 + (nt / 64) * 2 * cpt * 1024 <= 160 * 1024 ? cpt : 0;
+}
+constexpr int fold_stage_bytes(int bi, int bj, int nt, int nslot) { return (nt / 64) * 2 * fold_tiles(bi, bj, nt, nslot) * 1024; }
 
 template <int BI, int BJ, int WI, int WJ, int NSLOT, bool XK, bool YK, class CT, class DT, bool F16ACC>
 __global__ __launch_bounds__(WI *WJ * 64) __attribute__((amdgpu_waves_per_eu(waves_per_simd(BI, BJ, WI *WJ * 64))))
@@ -421,8 +448,60 @@ void k_gemm_tiled(tiled_params p)
     // younger pairs stay in flight across the barrier).  On the last trip
     // nothing new lands; its odd step reads another slot's stale bytes into
     // registers nobody uses.
+
+    // Folding C.  With alpha == 1 the C operand is added into the accumulators
+    // during the last NCT trips of the loop, CPT MFMA tiles per trip, so that
+    // the memory system delivers C while the matrix cores run and the epilogue
+    // only stores.  Group g (tiles g*CPT..) is requested at the end of a trip
+    // with direct-to-LDS loads: lane l fetches the 16 bytes it will own, so the
+    // wavefront's staging buffer is read back lane-contiguously by the same
+    // wavefront and needs no barrier of its own.  These loads are the youngest
+    // when the next trip waits, which lets exactly them stay in flight; the
+    // wait of the trip after that covers them (they are older than everything
+    // it leaves in flight), and that trip adds the group in: C has two trips to
+    // arrive from HBM.  Two staging buffers alternate.  Tiles are taken in the
+    // order of their addresses: 16 rows (64 bytes, the instruction's offset
+    // field) further down a column block, then the next 16 columns.  The
+    // accumulators are registers, so the folding trips are unrolled.
+    constexpr int CPT = fold_tiles(BI, BJ, NT, NSLOT);
+    constexpr bool CAN_FOLD = !F16ACC && __is_same(CT, float) && CPT > 0;
+    constexpr int NTILE = TI * TJ;
+    constexpr int NCT = CAN_FOLD ? NTILE / CPT : 1;  // groups, and trips that fold
+    static_assert(!CAN_FOLD || (TI % CPT == 0 && NCT >= 2), "fold groups");
+    bool fold_c = false;
+    if constexpr (CAN_FOLD) fold_c = p.use_c && !p.c_trans && p.alpha == 1.0f && NP > NCT;
+    const unsigned cstage = (unsigned)(uintptr_t)lds + (unsigned)(NSLOT * SLOT) + (unsigned)wave * (2u * CPT * 1024u);
+    const char *cnext = (const char *)(C + (long)j0 * p.ldc + i0);
+    const unsigned coff = 4u * (unsigned)((wj * WTJ + r) * (int)p.ldc + wi * WTI + 4 * q);
+    auto fold_request = [&]<int G>(std::integral_constant<int, G>) {
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            (([&] {
+                 constexpr int a = (G * CPT + U) % TI;
+                 lds_dma16_imm<64 * a>(cnext, coff, cstage + (unsigned)(((G & 1) * CPT + U) * 1024));
+                 if constexpr (a == TI - 1) cnext += 64 * p.ldc;
+             }()),
+             ...);
+        }(std::make_integer_sequence<int, CPT>{});
+    };
+    float4_t cfold[CPT > 0 ? CPT : 1];
+    auto fold_fetch = [&]<int G>(std::integral_constant<int, G>) {
+#pragma unroll
+        for (int u = 0; u < CPT; u++)
+            cfold[u] = *(MIW_LDS const float4_t *)(lds + NSLOT * SLOT + wave * (2 * CPT * 1024) +
+                                                   ((G & 1) * CPT + u) * 1024 + lane * 16);
+    };
+    auto fold_add = [&]<int G>(std::integral_constant<int, G>) {
+#pragma unroll
+        for (int u = 0; u < CPT; u++) {
+            const int a = (G * CPT + u) % TI, b = (G * CPT + u) / TI;
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[a][b][e] = __builtin_fmaf(p.beta, cfold[u][e], acc[a][b][e]);
+        }
+    };
+
     int rslot = 0;
-    for (int pr = 0; pr < NP; pr++) {
+    const int NPM = fold_c ? NP - NCT : NP;
+    for (int pr = 0; pr < NPM; pr++) {
         step(f0, f1, rslot, second_half, dma_begin, dma_begin);
         wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
         rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
@@ -430,7 +509,36 @@ void k_gemm_tiled(tiled_params p)
         step(f1, f0, rslot, first_half, dma_begin, dma_end);
         end_request();
     }
+    if constexpr (CAN_FOLD) {
+        if (fold_c) {
+            [&]<int... G>(std::integer_sequence<int, G...>) {
+                (([&] {
+                     step(f0, f1, rslot, second_half, dma_begin, dma_begin);
+                     wait_loads_and_barrier<(NSLOT - 2) * LPAIR + (G > 0 ? CPT : 0)>();
+                     rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
+                     if constexpr (G > 1) fold_fetch(std::integral_constant<int, G - 2>{});
+                     __builtin_amdgcn_sched_barrier(0);
+                     begin_request();
+                     step(f1, f0, rslot, first_half, dma_begin, dma_end);
+                     end_request();
+                     if constexpr (G > 1) fold_add(std::integral_constant<int, G - 2>{});
+                     __builtin_amdgcn_sched_barrier(0);
+                     fold_request(std::integral_constant<int, G>{});
+                     __builtin_amdgcn_sched_barrier(0);
+                 }()),
+                 ...);
+            }(std::make_integer_sequence<int, NCT>{});
+        }
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may outlive the workgroup's LDS
+    if constexpr (CAN_FOLD) {
+        if (fold_c) {
+            fold_fetch(std::integral_constant<int, NCT - 2>{});
+            fold_add(std::integral_constant<int, NCT - 2>{});
+            fold_fetch(std::integral_constant<int, NCT - 1>{});
+            fold_add(std::integral_constant<int, NCT - 1>{});
+        }
+    }
 
     // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
     auto epilogue = [&](bool with_c, bool trans) {
@@ -457,7 +565,7 @@ void k_gemm_tiled(tiled_params p)
                 }
             }
     };
-    if (F16ACC || !p.use_c) epilogue(false, false);
+    if (F16ACC || !p.use_c || fold_c) epilogue(false, false);
     else if (p.c_trans) epilogue(true, true);
     else epilogue(true, false);
 }
@@ -560,11 +668,12 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
 
     const void *fn = pick_kernel(i, xk, yk, c_type, d_type, f16acc);
     if (!fn) return hipErrorInvalidValue;
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, v.lds_bytes);
+    const int lds_bytes = v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return e;
     void *args[] = {&p};
     dim3 grid((unsigned)(p.tiles_i * p.tiles_j), (unsigned)g.batch);
-    return hipLaunchKernel(fn, grid, dim3((unsigned)(v.wm * v.wn * 64)), args, (size_t)v.lds_bytes, s);
+    return hipLaunchKernel(fn, grid, dim3((unsigned)(v.wm * v.wn * 64)), args, (size_t)lds_bytes, s);
 }
 
 // ------------------------------------------------------------ probes -------
