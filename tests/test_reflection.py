@@ -67,4 +67,4 @@ def test_tiled_kernels_keep_spills_out_of_the_steady_state(miw):
         assert per_trip >= 2 and not [l for l in body if re.match(r"\s*scratch_", l)], name
         if "256, 256, 2, 2, 2" in name:
             continue    # 256 accumulators per lane: the 4-wavefront tile spills around its loop
-        assert sum(1 for l in lines[mfma[0]:mfma[-1]] if re.match(r"\s*scratch_", l)) <= 32, name
+        assert sum(1 for l in lines[mfma[0]:mfma[-1]] if re.match(r"\s*scratch_", l)) <= 48, name
