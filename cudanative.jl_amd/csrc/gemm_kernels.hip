@@ -590,6 +590,7 @@ static const tiled_variant g_variants[] = {
     {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2},
     {"tile256x128_w2x2", 256, 128, KGRAN, 2, 2, 3, 3 * (256 + 128) * KGRAN * 2},
     {"tile128x256_w2x2", 128, 256, KGRAN, 2, 2, 3, 3 * (128 + 256) * KGRAN * 2},
+    {"tile128x128_w2x4_s4", 128, 128, KGRAN, 2, 4, 4, 4 * (128 + 128) * KGRAN * 2},
     {"tile128x128_w2x2_s4", 128, 128, KGRAN, 2, 2, 4, 4 * (128 + 128) * KGRAN * 2},
     {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2},
     {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, 4, 4 * (64 + 64) * KGRAN * 2},
@@ -635,9 +636,10 @@ static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, 
         case 1: return pick_types<256, 256, 2, 2, 2>(xk, yk, c_type, d_type, f16acc);
         case 2: return pick_types<256, 128, 2, 2, 3>(xk, yk, c_type, d_type, f16acc);
         case 3: return pick_types<128, 256, 2, 2, 3>(xk, yk, c_type, d_type, f16acc);
-        case 4: return pick_types<128, 128, 2, 2, 4>(xk, yk, c_type, d_type, f16acc);
-        case 5: return pick_types<128, 128, 2, 2, 2>(xk, yk, c_type, d_type, f16acc);
-        case 6: return pick_types<64, 64, 2, 2, 4>(xk, yk, c_type, d_type, f16acc);
+        case 4: return pick_types<128, 128, 2, 4, 4>(xk, yk, c_type, d_type, f16acc);
+        case 5: return pick_types<128, 128, 2, 2, 4>(xk, yk, c_type, d_type, f16acc);
+        case 6: return pick_types<128, 128, 2, 2, 2>(xk, yk, c_type, d_type, f16acc);
+        case 7: return pick_types<64, 64, 2, 2, 4>(xk, yk, c_type, d_type, f16acc);
     }
     return nullptr;
 }
