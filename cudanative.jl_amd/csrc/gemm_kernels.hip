@@ -231,13 +231,14 @@ constexpr int waves_per_simd(int bi, int bj, int nt) { return bi * bj / nt <= 12
 // (0: the variant does not fold).  Folding needs the accumulators in ordinary
 // VGPRs, at most one pair in flight across a barrier, and LDS room for two
 // staging buffers of that many 1 KiB tiles per wavefront.  Only the 8-wavefront
-// tile folds: the 4-wavefront kernels issue half as many loads per thread again
+// tiles fold: the 4-wavefront kernels issue half as many loads per thread again
 // and the register allocator answers the unrolled tail with spills.
 constexpr int fold_tiles(int bi, int bj, int nt, int nslot)
 {
     if (waves_per_simd(bi, bj, nt) < 2 || nslot > 3 || nt != 512) return 0;
-    const int cpt = 2;
-    return nslot * (bi + bj) * KGRAN * 2 + (nt / 64) * 2 * cpt * 1024 <= 160 * 1024 ? cpt : 0;
+    for (int cpt = 2; cpt >= 1; cpt--)
+        if (nslot * (bi + bj) * KGRAN * 2 + (nt / 64) * 2 * cpt * 1024 <= 160 * 1024) return cpt;
+    return 0;
 }
 constexpr int fold_stage_bytes(int bi, int bj, int nt, int nslot) { return (nt / 64) * 2 * fold_tiles(bi, bj, nt, nslot) * 1024; }
 
@@ -588,8 +589,8 @@ static const tiled_variant g_variants[] = {
     // name                    bm   bn  bk     wm wn slots lds
     {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2},
     {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2},
-    {"tile256x128_w2x2", 256, 128, KGRAN, 2, 2, 3, 3 * (256 + 128) * KGRAN * 2},
-    {"tile128x256_w2x2", 128, 256, KGRAN, 2, 2, 3, 3 * (128 + 256) * KGRAN * 2},
+    {"tile256x128_w4x2", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2},
+    {"tile128x256_w2x4", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2},
     {"tile128x128_w2x4_s4", 128, 128, KGRAN, 2, 4, 4, 4 * (128 + 128) * KGRAN * 2},
     {"tile128x128_w2x2_s4", 128, 128, KGRAN, 2, 2, 4, 4 * (128 + 128) * KGRAN * 2},
     {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2},
@@ -634,8 +635,8 @@ static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, 
     switch (i) {
         case 0: return pick_types<256, 256, 2, 4, 2>(xk, yk, c_type, d_type, f16acc);
         case 1: return pick_types<256, 256, 2, 2, 2>(xk, yk, c_type, d_type, f16acc);
-        case 2: return pick_types<256, 128, 2, 2, 3>(xk, yk, c_type, d_type, f16acc);
-        case 3: return pick_types<128, 256, 2, 2, 3>(xk, yk, c_type, d_type, f16acc);
+        case 2: return pick_types<256, 128, 4, 2, 3>(xk, yk, c_type, d_type, f16acc);
+        case 3: return pick_types<128, 256, 2, 4, 3>(xk, yk, c_type, d_type, f16acc);
         case 4: return pick_types<128, 128, 2, 4, 4>(xk, yk, c_type, d_type, f16acc);
         case 5: return pick_types<128, 128, 2, 2, 4>(xk, yk, c_type, d_type, f16acc);
         case 6: return pick_types<128, 128, 2, 2, 2>(xk, yk, c_type, d_type, f16acc);

@@ -133,16 +133,19 @@ def test_tiled_variants_agree_bitwise(gpu, orc):
     assert np.array_equal(_run(gpu, orc, g, A, B, C, variant=1).view(np.uint32), outs[0].view(np.uint32))
 
 
-# K long enough (more than 16 LDS slots' worth) for the 8-wavefront 256x256 kernel to add C into
-# its accumulators during the last trips of its loop instead of in the epilogue.
+# K long enough (more than 16 LDS slots' worth) for the 8-wavefront 256x256, 256x128 and 128x256
+# kernels to add C into their accumulators during the last trips of the loop instead of in the epilogue.
 
 @pytest.mark.parametrize("al,bl,dl", itertools.product((0, 1), repeat=3))
 @pytest.mark.parametrize("K", [17 * 64, 20 * 64])
 def test_c_folded_into_the_loop_exact_on_integers(gpu, orc, al, bl, dl, K):
-    g = orc.GemmDesc(M=512, N=256, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, beta=-2.0)
-    A, B, C = _inputs(orc, g, 500 + K, ints=True)
-    D = _run(gpu, orc, g, A, B, C, variant=1)
-    assert np.array_equal(D, orc.gemm(g, A, B, C)), (al, bl, dl, K)
+    folding = [v for v in _variants(gpu) if v["waves"][0] * v["waves"][1] == 8 and v["stages"] <= 3]
+    assert [v["block"][:2] for v in folding] == [(256, 256), (256, 128), (128, 256)]
+    for v in folding:
+        g = orc.GemmDesc(M=512, N=256, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, beta=-2.0)
+        A, B, C = _inputs(orc, g, 500 + K + v["id"], ints=True)
+        D = _run(gpu, orc, g, A, B, C, variant=v["id"])
+        assert np.array_equal(D, orc.gemm(g, A, B, C)), (v["name"], al, bl, dl, K)
 
 
 def test_c_folded_into_the_loop_matches_the_epilogue_path(gpu, orc):
@@ -155,6 +158,8 @@ def test_c_folded_into_the_loop_matches_the_epilogue_path(gpu, orc):
     ref = orc.gemm_f64(g, A, B, C)
     folded = _run(gpu, orc, g, A, B, C, variant=1, prefill=5.0)
     assert orc.normalized_error(g, folded, ref) <= TIGHT_F32
+    for v in (3, 4):
+        assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C, variant=v, prefill=5.0), ref) <= TIGHT_F32
     other = _run(gpu, orc, g, A, B, C, variant=2, prefill=5.0)           # 4 wavefronts: C in the epilogue
     assert orc.normalized_error(g, other, ref) <= TIGHT_F32
     assert np.max(np.abs(folded.astype(np.float64) - other)) <= 4e-7 * np.abs(ref).max()   # padding: 5.0 in both
