@@ -26,9 +26,9 @@ PEAK_HBM_GBS = 8000.0
 # each scaled by what the counter reads for the library's copy kernel on 256 MiB; the summaries
 # and commands are under profiles/.  Configurations without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    "c2": int((256.1 + 69.5) * 2 ** 20),   # profiles/gemm_tiled_256x256_4096cubed_f32acc.md
+    "c2": int((256.4 + 69.4) * 2 ** 20),   # profiles/gemm_tiled_256x256_4096cubed_f32acc.md
     "c3": int((56.1 + 8.0) * 2 ** 20),     # profiles/gemm_tiled_128x128_2048cubed_f16acc.md
-    "c4": int((160.1 + 33.6) * 2 ** 20),   # profiles/gemm_tiled_256x128_8192x1024x4096_mixed_layout.md
+    "c4": int((160.3 + 38.5) * 2 ** 20),   # profiles/gemm_tiled_256x128_8192x1024x4096_mixed_layout.md
     "c5": int((64.1 + 32.0) * 2 ** 20),    # profiles/gemm_tiled_128x128_batched_512x128cubed.md
 }
 
