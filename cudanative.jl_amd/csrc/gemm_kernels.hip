@@ -482,7 +482,8 @@ void k_gemm_tiled(tiled_params p)
     constexpr int NCT = CAN_FOLD ? NTILE / CPT : 1;  // groups, and trips that fold
     static_assert(!CAN_FOLD || (TI % CPT == 0 && NCT >= 2), "fold groups");
     bool fold_c = false;
-    if constexpr (CAN_FOLD) fold_c = p.use_c && !p.c_trans && p.alpha == 1.0f && NP > NCT;
+    // (the lane offset into the tile of C is kept in 32 bits)
+    if constexpr (CAN_FOLD) fold_c = p.use_c && !p.c_trans && p.alpha == 1.0f && NP > NCT && p.ldc < (1l << 22);
     const unsigned cstage = (unsigned)(uintptr_t)lds + (unsigned)(NSLOT * SLOT) + (unsigned)wave * (2u * CPT * 1024u);
     const char *cnext = (const char *)(C + (long)j0 * p.ldc + i0);
     const unsigned coff = 4u * (unsigned)((wj * WTJ + r) * (int)p.ldc + wi * WTI + 4 * q);
