@@ -177,6 +177,18 @@ def test_c_folded_into_the_loop_matches_the_epilogue_path(gpu, orc):
     assert orc.normalized_error(g4, _run(gpu, orc, g4, A, B, C, variant=1), orc.gemm_f64(g4, A, B, C)) <= TIGHT_F32
 
 
+def test_c_and_d_may_be_one_buffer(gpu, orc):
+    """In place: D = A*B + beta*D.  Every workgroup reads its tile of C before it stores that tile."""
+    for variant, (M, N, K) in ((1, (512, 256, 1600)), (1, (256, 256, 256)), (7, (256, 128, 192)), (0, (48, 80, 64))):
+        g = orc.GemmDesc(M=M, N=N, K=K, beta=0.5)
+        A, B, C = _inputs(orc, g, 900 + variant + K)
+        dA, dB, dD = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(C.copy())
+        desc = gpu.GEMM.make_desc(M, N, K, beta=0.5, variant=variant)
+        gpu.GEMM.gemm(dA, dB, dD, dD, desc)
+        gpu.synchronize()
+        assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32, (variant, M, N, K)
+
+
 def test_ragged_sizes_fall_back_to_fragment_ops(gpu, orc):
     # multiples of 16 that no LDS tile divides, padded leading dimensions, odd batch strides
     g = orc.GemmDesc(M=80, N=112, K=176, lda=88, ldb=200, ldc=96, ldd=104, batch=3,
