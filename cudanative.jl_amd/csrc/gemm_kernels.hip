@@ -414,6 +414,12 @@ void k_gemm_tiled(tiled_params p)
         [&]<int... Mi>(std::integer_sequence<int, Mi...>) {
             (([&] {
                  constexpr int m = Mi;
+                 // The SIMD issues from its oldest ready wavefront first, which lets one of its two
+                 // wavefronts run a whole step ahead and then stand at the barrier while the other
+                 // works alone; raising the priority over the first half of every step makes the
+                 // two take turns.
+                 if constexpr (NMFMA >= 8 && m == 0) __builtin_amdgcn_s_setprio(1);
+                 if constexpr (NMFMA >= 8 && m == NMFMA / 2) __builtin_amdgcn_s_setprio(0);
                  if constexpr (m < NUNIT) fetch_unit(nxt, xs, std::integral_constant<int, m>{}, h);
                  constexpr int a = m / TJ, b = m % TJ;
                  acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.x[a], cur.y[b], acc[a][b], 0, 0, 0);
