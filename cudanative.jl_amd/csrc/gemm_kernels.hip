@@ -460,13 +460,6 @@ void k_gemm_tiled(tiled_params p)
         (fetch_unit(f0, lds, std::integral_constant<int, U>{}, first_half), ...);
     }(std::make_integer_sequence<int, NUNIT>{});
 
-    // Trip pr: step 2pr (second half of pair pr's slot is fetched; nothing to
-    // request yet: the slot is still being read), barrier (pair pr+1 has
-    // landed, pair pr's slot is free), step 2pr+1 (first half of pair pr+1 is
-    // fetched while pair pr+NSLOT is requested into the freed slot; NSLOT-2
-    // younger pairs stay in flight across the barrier).  On the last trip
-    // nothing new lands; its odd step reads another slot's stale bytes into
-    // registers nobody uses.
 
     // Folding C.  With alpha == 1 the C operand is added into the accumulators
     // during the last NCT trips of the loop, CPT MFMA tiles per trip, so that
@@ -519,6 +512,13 @@ void k_gemm_tiled(tiled_params p)
         }
     };
 
+    // Trip pr: step 2pr (second half of pair pr's slot is fetched; nothing to
+    // request yet: the slot is still being read), barrier (pair pr+1 has
+    // landed, pair pr's slot is free), step 2pr+1 (first half of pair pr+1 is
+    // fetched while pair pr+NSLOT is requested into the freed slot; NSLOT-2
+    // younger pairs stay in flight across the barrier).  On the last trip
+    // nothing new lands; its odd step reads another slot's stale bytes into
+    // registers nobody uses.
     int rslot = 0;
     const int NPM = fold_c ? NP - NCT : NP;
     for (int pr = 0; pr < NPM; pr++) {
