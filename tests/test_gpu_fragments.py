@@ -332,7 +332,7 @@ def test_example_low_level(gpu):
 
 
 def test_config1_golden_fixture(gpu, orc):
-    # BASELINE config 1: single fragment, seed 0, normalized error <= 1e-3 (fp32 accumulate)
+    # benchmark configuration 1: single fragment, seed 0, normalized error <= 1e-3 (fp32 accumulate)
     z = np.load(os.path.join(GOLD, "c1_fragment_seed0.npz"))
     W = gpu.WMMA
     a_dev, b_dev, c_dev = gpu.DeviceArray(z["A"]), gpu.DeviceArray(z["B"]), gpu.DeviceArray(z["C"])

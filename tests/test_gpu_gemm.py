@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 F16, F32 = np.float16, np.float32
 
-# tolerances of BASELINE's north star: max|D - Dref| / max|Dref|
+# tolerances of the benchmark definition: max|D - Dref| / max|Dref|
 TOL_F32ACC = 1e-3
 TOL_F16ACC = 1e-2
 # what fp32 accumulation actually achieves; a wrong tile or a dropped k-slice is ~1e-1
@@ -322,7 +322,7 @@ def test_f16acc_alpha_beta(gpu, orc):
         _run(gpu, orc, g, A, B, C, acc_type=F16, variant=len(_variants(gpu)) - 1)
 
 
-# ------------------------------------------------------------- BASELINE configs ---
+# ------------------------------------------------------------- benchmark configurations ---
 
 def _sampled_error(orc, g, A, B, C, D, rows, bt=0):
     """normalized error over a sample of full rows of D (D_ref rows in float64 by numpy)."""
