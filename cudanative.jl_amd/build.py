@@ -10,7 +10,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmiwmma.so")
-SOURCES = ["capi.hip", "frag_kernels.hip", "gemm_kernels.hip"]
+SOURCES = ["gemm_tile_256x256_w2x4.hip", "gemm_tile_256x128.hip", "gemm_tile_256x256_w2x2.hip", "gemm_tile_small.hip",
+           "capi.hip", "frag_kernels.hip", "gemm_kernels.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",

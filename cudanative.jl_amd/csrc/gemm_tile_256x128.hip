@@ -1,0 +1,16 @@
+// Instances of the tiled GEMM kernel for one tile family (see gemm_tiled.hpp).
+#include "gemm_tiled.hpp"
+
+namespace miw {
+
+const void *tiled_kernel_256x128_w4x2(bool xk, bool yk, int c_type, int d_type, bool f16acc)
+{
+    return pick_types<256, 128, 4, 2, 3>(xk, yk, c_type, d_type, f16acc);
+}
+
+const void *tiled_kernel_128x256_w2x4(bool xk, bool yk, int c_type, int d_type, bool f16acc)
+{
+    return pick_types<128, 256, 2, 4, 3>(xk, yk, c_type, d_type, f16acc);
+}
+
+}  // namespace miw
