@@ -90,6 +90,7 @@ def main():
                     help="untimed launches before the warm-up steps, until the GPU's power management has "
                          "raised the clocks from idle (the first ~250 launches after idle run up to 20 %% slower)")
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--rotate", type=int, default=1, help="cycle the timed launches through N copies of the operands")
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -150,13 +151,18 @@ def main():
         for _ in range(50):
             G.gemm(dA, dB, dC, dD, desc)
         m.synchronize()
-    for _ in range(args.warmup):
-        G.gemm(dA, dB, dC, dD, desc)
+    # --rotate N: the timed launches cycle through N copies of every operand, so that a working
+    # set smaller than the 256 MiB Infinity Cache is not served from it ("hot" is the default)
+    sets = [(dA, dB, dC, dD)]
+    for _ in range(1, max(args.rotate, 1)):
+        sets.append((m.DeviceArray(A), m.DeviceArray(B), m.DeviceArray(C), m.DeviceArray.undef(ct, batch * M * N)))
+    for i in range(args.warmup):
+        G.gemm(*sets[i % len(sets)], desc)
     m.synchronize()
     t0 = time.perf_counter()
     m._lib.check(lib.miw_event_record(ev0, None))
-    for _ in range(args.steps):
-        G.gemm(dA, dB, dC, dD, desc)
+    for i in range(args.steps):
+        G.gemm(*sets[i % len(sets)], desc)
     m._lib.check(lib.miw_event_record(ev1, None))
     m.synchronize()
     wall = time.perf_counter() - t0
@@ -201,6 +207,7 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 in, f16 accumulate" if half else "f16 in, f32 accumulate", "data": "synthetic",
         "config": {"workload": cfg["workload"], "variant": vinfo["name"], "batch": batch,
+                   "operand_sets": len(sets),
                    "algorithmic_flop": flops, "algorithmic_bytes": abytes,
                    "normalized_error_sampled": err, "tolerance": 1e-2 if half else 1e-3,
                    "pct_of_fp16_dense_peak": 100.0 * value / PEAK_F16_DENSE_TFLOPS,
