@@ -189,6 +189,38 @@ def test_c_and_d_may_be_one_buffer(gpu, orc):
         assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32, (variant, M, N, K)
 
 
+def test_seeded_sweep_over_variants_layouts_and_scalars(gpu, orc):
+    """300 seeded draws of (tiled variant, tile counts, K from one slot's worth to past the point
+    where C is folded in, layouts of all four matrices, C/D types, alpha, beta, use_c, batch,
+    padded leading dimensions, integer or uniform data), each against float64."""
+    rng = np.random.default_rng(2024)
+    vs = [v for v in _variants(gpu) if not v["fragment_ops"]]
+    for case in range(300):
+        v = vs[rng.integers(0, len(vs))]
+        bm, bn, _ = v["block"]
+        dl = int(rng.integers(0, 2))
+        mi, ni = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        M, N = (bm * mi, bn * ni) if dl == 1 else (bn * ni, bm * mi)      # bm tiles D's contiguous dimension
+        K = 64 * int(rng.choice([1, 2, 3, 8, 16, 17, 18, 19, 24, 33]))
+        al, bl = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        cl = dl if rng.random() < 0.8 else 1 - dl
+        alpha = 1.0 if rng.random() < 0.7 else float(rng.choice([0.5, -2.0]))
+        beta = float(rng.choice([1.0, 0.0, -0.5, 2.0]))
+        use_c = int(rng.random() < 0.85)
+        batch = int(rng.choice([1, 1, 2, 3]))
+        ct, dt = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        pad = int(rng.choice([0, 0, 8, 16]))
+        g0 = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl).resolved()
+        g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=ct, d_type=dt,
+                         alpha=alpha, beta=beta, use_c=use_c, batch=batch, lda=g0.lda + pad, ldb=g0.ldb + pad,
+                         ldc=g0.ldc + pad, ldd=g0.ldd + pad)
+        A, B, C = _inputs(orc, g, int(rng.integers(0, 10000)), ints=bool(rng.random() < 0.5))
+        D = _run(gpu, orc, g, A, B, C if use_c else None, variant=v["id"], prefill=7.0)
+        err = orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C))
+        assert err <= (TIGHT_F32 if dt == orc.F32 else 6e-4), (case, v["name"], M, N, K, al, bl, cl, dl, alpha, beta,
+                                                              use_c, batch, ct, dt, pad, err)
+
+
 def test_ragged_sizes_fall_back_to_fragment_ops(gpu, orc):
     # multiples of 16 that no LDS tile divides, padded leading dimensions, odd batch strides
     g = orc.GemmDesc(M=80, N=112, K=176, lda=88, ldb=200, ldc=96, ldd=104, batch=3,
