@@ -164,6 +164,12 @@ def test_abi_rejects_bad_arguments_without_touching_the_gpu(miw):
     assert lib.miw_frag_elems_per_lane(L.ACCUMULATOR, L.F32) == 4
     assert lib.miw_frag_image_bytes(L.MATRIX_A, L.F16) == 512 and lib.miw_frag_image_bytes(L.ACCUMULATOR, L.F32) == 1024
 
+    f1 = (ctypes.c_float * 1)()
+    assert lib.miw_launch_overhead_probe(0, 1000, f1, f1) == L.ERR_INVALID_VALUE
+    assert lib.miw_launch_overhead_probe(1, 2000, f1, f1) == L.ERR_INVALID_VALUE
+    assert lib.miw_launch_overhead_probe(1, 1000, None, f1) == L.ERR_INVALID_VALUE
+    assert lib.miw_mfma_peak_probe(0, ctypes.byref(ctypes.c_double()), None) == L.ERR_INVALID_VALUE
+
     G = miw.GEMM
     d = G.make_desc(100, 64, 64)
     assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_SHAPE
