@@ -93,6 +93,8 @@ def main():
     ap.add_argument("--rotate", type=int, default=1, help="cycle the timed launches through N copies of the operands")
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="only run the matrix-core power probe (zero and random operands) and print its line")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="instead of the GEMM, launch the library's plain copy kernel on MIB MiB a few times "
                          "(calibrates the FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -106,6 +108,14 @@ def main():
     from oracle import oracle as orc
     m = load_package()
     m.init(0)
+    if args.mfma_probe:
+        out = {}
+        for name, rnd in (("zero_operands", False), ("random_operands", True)):
+            m.mfma_power_probe(5000, rnd)
+            tf, mhz = m.mfma_power_probe(40000, rnd)
+            out[name] = {"tflops": tf, "shader_mhz": mhz, "frac_of_peak": tf / PEAK_F16_DENSE_TFLOPS}
+        print(json.dumps({"mfma_power_probe": out, "instruction": "v_mfma_f32_16x16x32_f16", "unit": "TFLOP/s"}))
+        return
     if args.copy_probe:
         n = args.copy_probe << 20
         src, dst = m.DeviceArray.undef(np.uint8, n), m.DeviceArray.undef(np.uint8, n)

@@ -47,6 +47,13 @@ def functional():
         return False
 
 
+def mfma_power_probe(iters=20000, random_operands=True):
+    """(TFLOP/s, shader MHz) of the matrix cores alone on operands that change every k-step."""
+    t, f = _ctypes.c_double(), _ctypes.c_double()
+    _lib.check(_lib.load().miw_mfma_power_probe(iters, int(bool(random_operands)), _ctypes.byref(t), _ctypes.byref(f), None))
+    return t.value, f.value
+
+
 def mfma_peak_tflops(iters=20000):
     v = _ctypes.c_double()
     _lib.check(_lib.load().miw_mfma_peak_probe(iters, _ctypes.byref(v), None))

@@ -133,6 +133,7 @@ SIGNATURES = {
     "miw_gemm_acc_chunk": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
     "miw_gemm_bench": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _vp, _i, _i, ctypes.POINTER(_f)]),
     "miw_launch_overhead_probe": (_i, [_i, _i, ctypes.POINTER(_f), ctypes.POINTER(_f)]),
+    "miw_mfma_power_probe": (_i, [_i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), _vp]),
     "miw_mfma_peak_probe": (_i, [_i, ctypes.POINTER(ctypes.c_double), _vp]),
     "miw_copy_probe": (_i, [_vp, _vp, _sz, _vp]),
     "miw_kernel_count": (_i, []),

@@ -566,6 +566,49 @@ int miw_launch_overhead_probe(int iters, int threads, float *cpu_us, float *gpu_
     return 0;
 }
 
+int miw_mfma_power_probe(int iters, int random_operands, double *tflops, double *shader_mhz, void *stream)
+{
+    if (!tflops || !shader_mhz || iters < 1) return fail(MIW_ERR_INVALID_VALUE, "mfma_power_probe: bad arguments");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    int wall_khz = 0;
+    HIP_TRY(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, dev));
+    const int blocks = prop.multiProcessorCount;  // one 8-wavefront workgroup per CU
+    float *sink = nullptr;
+    long long *ticks = nullptr;
+    HIP_TRY(hipMalloc((void **)&sink, 4));
+    hipError_t he = hipMalloc((void **)&ticks, sizeof(long long) * 2 * blocks);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipStream_t s = as_stream(stream);
+    const float scale = random_operands ? 1.0f : 0.0f;
+    if (he == hipSuccess) he = hipEventCreate(&e0);
+    if (he == hipSuccess) he = hipEventCreate(&e1);
+    if (he == hipSuccess) he = miw::launch_mfma_power(blocks, iters / 4 + 1, scale, sink, ticks, s);  // warm-up
+    if (he == hipSuccess) he = hipEventRecord(e0, s);
+    if (he == hipSuccess) he = miw::launch_mfma_power(blocks, iters, scale, sink, ticks, s);
+    if (he == hipSuccess) he = hipEventRecord(e1, s);
+    if (he == hipSuccess) he = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+    std::vector<long long> host(2 * (size_t)blocks);
+    if (he == hipSuccess) he = hipMemcpy(host.data(), ticks, sizeof(long long) * host.size(), hipMemcpyDeviceToHost);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    (void)hipFree(ticks);
+    if (he != hipSuccess) return hip_fail(he, "mfma_power_probe");
+    // per wavefront and iteration: 4 sets x 16 MFMAs of 16*16*32*2 flop
+    const double flop = (double)blocks * 8.0 * (double)iters * 64.0 * 16384.0;
+    *tflops = flop / ((double)ms * 1e-3) / 1e12;
+    double mhz = 0.0;
+    for (int b = 0; b < blocks; b++)
+        mhz += (double)host[2 * b] / ((double)host[2 * b + 1] / ((double)wall_khz * 1e3)) / 1e6;
+    *shader_mhz = mhz / blocks;
+    return 0;
+}
+
 int miw_mfma_peak_probe(int iters, double *tflops, void *stream)
 {
     if (!tflops || iters < 1) return fail(MIW_ERR_INVALID_VALUE, "mfma_peak_probe: bad arguments");

@@ -129,6 +129,55 @@ hipError_t launch_mfma_peak(int blocks, int iters, float *sink, hipStream_t s)
     return hipGetLastError();
 }
 
+// The same chain on operands that change every k-step (four register-resident sets of four A
+// and four B fragments, pseudo-random or all zero), as a GEMM's do: what the matrix cores
+// sustain under the power cap.  Each workgroup reports its shader-clock and wall-clock ticks.
+__device__ inline unsigned probe_hash(unsigned x)
+{
+    x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+    return x;
+}
+
+__global__ __launch_bounds__(512) void k_mfma_power(int iters, float scale, float *sink, long long *ticks)
+{
+    constexpr int NSET = 4;
+    half8_t a[NSET][4], b[NSET][4];
+    for (int s = 0; s < NSET; s++)
+        for (int i = 0; i < 4; i++)
+            for (int e = 0; e < 8; e++) {
+                const unsigned seed = ((blockIdx.x * 512u + threadIdx.x) * 32u + s * 8u + i) * 16u + e;
+                a[s][i][e] = (half_t)(scale * ((float)(probe_hash(2 * seed + 1) & 0xffff) / 32768.f - 1.f));
+                b[s][i][e] = (half_t)(scale * ((float)(probe_hash(2 * seed + 2) & 0xffff) / 32768.f - 1.f));
+            }
+    float4_t acc[4][4];
+    for (int i = 0; i < 4; i++)
+        for (int j = 0; j < 4; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const long long c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; it++)
+#pragma unroll
+        for (int s = 0; s < NSET; s++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
+    const long long c1 = clock64(), w1 = wall_clock64();
+    float r = 0.f;
+    for (int i = 0; i < 4; i++)
+        for (int j = 0; j < 4; j++) r += acc[i][j][0] + acc[i][j][3];
+    if (r == 12345.678f) sink[0] = r;  // keeps the chain alive
+    if (threadIdx.x == 0) {
+        ticks[2 * blockIdx.x] = c1 - c0;
+        ticks[2 * blockIdx.x + 1] = w1 - w0;
+    }
+}
+
+hipError_t launch_mfma_power(int blocks, int iters, float scale, float *sink, long long *ticks, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_mfma_power, dim3((unsigned)blocks), dim3(512), 0, s, iters, scale, sink, ticks);
+    return hipGetLastError();
+}
+
 __global__ __launch_bounds__(256) void k_copy16(uint4_t *dst, const uint4_t *src, size_t n16)
 {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;

@@ -57,6 +57,9 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &p, int c_type, int d_type
 const void *tiled_kernel_symbol(int i);
 
 hipError_t launch_mfma_peak(int blocks, int iters, float *sink, hipStream_t s);
+// One 8-wavefront workgroup per block: 64 MFMAs per wavefront and iteration; ticks[2b], ticks[2b+1]:
+// shader-clock and wall-clock ticks workgroup b spent in the chain.
+hipError_t launch_mfma_power(int blocks, int iters, float scale, float *sink, long long *ticks, hipStream_t s);
 hipError_t launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s);
 
 }  // namespace miw

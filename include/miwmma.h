@@ -211,6 +211,11 @@ int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, cons
    of examples/peakflops.jl): measured TFLOP/s of the matrix cores alone. */
 int miw_mfma_peak_probe(int iters, double *tflops, void *stream);
 
+/* The same chain on operands that change every k-step (register-resident sets, all zero or
+   pseudo-random in [-1, 1)), one 8-wavefront workgroup per CU: what the matrix cores sustain
+   under the power cap, and the shader clock (MHz, mean over the CUs) they run at meanwhile. */
+int miw_mfma_power_probe(int iters, int random_operands, double *tflops, double *shader_mhz, void *stream);
+
 /* The raw-driver leg of the launch-overhead benchmark (test/perf/launch_overhead/cuda.c:60-80):
    iters times { record event; launch the dummy kernel with `threads` lanes; record event;
    synchronize }, all inside the library with no foreign-function hop; cpu_us[i] receives the

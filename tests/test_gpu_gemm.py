@@ -438,3 +438,6 @@ def test_bench_entry_reports_positive_times(gpu, orc):
     assert ms.shape == (5,) and np.all(ms > 0) and np.all(ms < 50)
     assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
     assert gpu.mfma_peak_tflops(2000) > 100
+    zero_tf, zero_mhz = gpu.mfma_power_probe(4000, random_operands=False)
+    rand_tf, rand_mhz = gpu.mfma_power_probe(4000, random_operands=True)
+    assert 100 < rand_tf <= zero_tf * 1.05 and 500 < rand_mhz <= zero_mhz * 1.05 < 2700    # random data never runs faster

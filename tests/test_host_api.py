@@ -169,6 +169,8 @@ def test_abi_rejects_bad_arguments_without_touching_the_gpu(miw):
     assert lib.miw_launch_overhead_probe(1, 2000, f1, f1) == L.ERR_INVALID_VALUE
     assert lib.miw_launch_overhead_probe(1, 1000, None, f1) == L.ERR_INVALID_VALUE
     assert lib.miw_mfma_peak_probe(0, ctypes.byref(ctypes.c_double()), None) == L.ERR_INVALID_VALUE
+    assert lib.miw_mfma_power_probe(0, 1, ctypes.byref(ctypes.c_double()), ctypes.byref(ctypes.c_double()), None) == L.ERR_INVALID_VALUE
+    assert lib.miw_mfma_power_probe(10, 1, None, ctypes.byref(ctypes.c_double()), None) == L.ERR_INVALID_VALUE
 
     G = miw.GEMM
     d = G.make_desc(100, 64, 64)
