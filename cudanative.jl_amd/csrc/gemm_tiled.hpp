@@ -450,7 +450,6 @@ void k_gemm_tiled(tiled_params p)
     constexpr std::integral_constant<int, 0> first_half{};
     constexpr std::integral_constant<int, 1> second_half{};
     constexpr std::integral_constant<int, 0> dma_begin{};
-    constexpr std::integral_constant<int, LPAIR / 2> dma_mid{};
     constexpr std::integral_constant<int, LPAIR> dma_end{};
 
     // Prologue: every slot requested, pair 0 published and its first fragments fetched.
@@ -460,7 +459,6 @@ void k_gemm_tiled(tiled_params p)
     [&]<int... U>(std::integer_sequence<int, U...>) {
         (fetch_unit(f0, lds, std::integral_constant<int, U>{}, first_half), ...);
     }(std::make_integer_sequence<int, NUNIT>{});
-
 
     // Folding C.  With alpha == 1 the C operand is added into the accumulators
     // during the last NCT trips of the loop, CPT MFMA tiles per trip, so that
