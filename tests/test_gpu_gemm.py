@@ -192,7 +192,8 @@ def test_c_and_d_may_be_one_buffer(gpu, orc):
 def test_seeded_sweep_over_variants_layouts_and_scalars(gpu, orc):
     """300 seeded draws of (tiled variant, tile counts, K from one slot's worth to past the point
     where C is folded in, layouts of all four matrices, C/D types, alpha, beta, use_c, batch,
-    padded leading dimensions, integer or uniform data), each against float64."""
+    padded leading dimensions, integer or uniform data), each against float64; a quarter of the
+    draws on variants that have one run the fp16-accumulate form, bit for bit against its model."""
     rng = np.random.default_rng(2024)
     vs = [v for v in _variants(gpu) if not v["fragment_ops"]]
     for case in range(300):
@@ -214,6 +215,19 @@ def test_seeded_sweep_over_variants_layouts_and_scalars(gpu, orc):
         g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=ct, d_type=dt,
                          alpha=alpha, beta=beta, use_c=use_c, batch=batch, lda=g0.lda + pad, ldb=g0.ldb + pad,
                          ldc=g0.ldc + pad, ldd=g0.ldd + pad)
+        if v["f16_accumulate"] and rng.random() < 0.25:
+            # fp16 accumulate on quarter-integers: every partial sum is exact in half, so the result
+            # must equal the chunked model bit for bit
+            h = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=orc.F16,
+                             d_type=orc.F16, beta=beta, use_c=use_c, batch=batch, lda=g.lda, ldb=g.ldb, ldc=g.ldc,
+                             ldd=g.ldd)
+            A, B, C = _inputs(orc, h, int(rng.integers(0, 10000)), ints=True)
+            A, B = (A / 4).astype(F16), (B / 4).astype(F16)
+            D = _run(gpu, orc, h, A, B, C if use_c else None, variant=v["id"], acc_type=F16, prefill=7.0)
+            model = orc.gemm_f16acc(h, 64, A, B, C)
+            live = model != 0                                 # the model leaves padding at zero
+            assert np.array_equal(D[live], model[live]), (case, v["name"], M, N, K, al, bl, cl, dl, beta, use_c, batch)
+            continue
         A, B, C = _inputs(orc, g, int(rng.integers(0, 10000)), ints=bool(rng.random() < 0.5))
         D = _run(gpu, orc, g, A, B, C if use_c else None, variant=v["id"], prefill=7.0)
         err = orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C))
