@@ -80,7 +80,7 @@ class GemmVariantInfo(ctypes.Structure):
         ("block_m", ctypes.c_int), ("block_n", ctypes.c_int), ("block_k", ctypes.c_int),
         ("waves_m", ctypes.c_int), ("waves_n", ctypes.c_int),
         ("stages", ctypes.c_int), ("lds_bytes", ctypes.c_int), ("fragment_ops", ctypes.c_int),
-        ("f16_accumulate", ctypes.c_int),
+        ("f16_accumulate", ctypes.c_int), ("pingpong", ctypes.c_int),
     ]
 
 
@@ -129,6 +129,7 @@ SIGNATURES = {
     "miw_gemm": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _vp]),
     "miw_gemm_variant_count": (_i, []),
     "miw_gemm_variant_info_get": (_i, [_i, ctypes.POINTER(GemmVariantInfo)]),
+    "miw_gemm_variant_supports": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(_i)]),
     "miw_gemm_pick_variant": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
     "miw_gemm_acc_chunk": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
     "miw_gemm_bench": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _vp, _i, _i, ctypes.POINTER(_f)]),

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -41,6 +42,16 @@ int hip_fail(hipError_t e, const char *what)
         if (e_ != hipSuccess) return hip_fail(e_, #expr); \
     } while (0)
 
+// Set by miw_init.  Entries that touch the device check it after their arguments: an invalid call
+// is reported as such with or without a device, a valid one needs the gfx950 check of miw_init.
+std::atomic<bool> g_initialized{false};
+#define REQUIRE_INIT(what)                                                                              \
+    do {                                                                                                \
+        if (!g_initialized.load(std::memory_order_acquire))                                             \
+            return fail(MIW_ERR_NOT_INITIALIZED, "%s: miw_init has not been called (it selects the device and " \
+                        "checks that it is a gfx950 part)", what);                                      \
+    } while (0)
+
 bool valid_layout(int l) { return l == MIW_ROW_MAJOR || l == MIW_COL_MAJOR; }
 bool valid_dtype(int t) { return t == MIW_F16 || t == MIW_F32; }
 bool valid_as(int a) { return a == MIW_AS_GENERIC || a == MIW_AS_GLOBAL || a == MIW_AS_SHARED; }
@@ -58,6 +69,7 @@ hipStream_t as_stream(void *s) { return (hipStream_t)s; }
 struct named_kernel {
     std::string name;
     const void *fn;
+    int launchable;  // 0: lookup and attribute queries only
 };
 
 std::vector<named_kernel> &registry()
@@ -66,10 +78,10 @@ std::vector<named_kernel> &registry()
         std::vector<named_kernel> v;
         for (int i = 0; i < miw::frag_kernel_count(); i++) {
             const char *n = miw::frag_kernel_name(i);
-            v.push_back({n, miw::frag_kernel_symbol(n)});
+            v.push_back({n, miw::frag_kernel_symbol(n), 1});
         }
         for (int i = 0; i < miw::tiled_variant_count(); i++)
-            v.push_back({std::string("gemm_") + miw::tiled_variant_at(i).name, miw::tiled_kernel_symbol(i)});
+            v.push_back({std::string("gemm_") + miw::tiled_variant_at(i).name, miw::tiled_kernel_symbol(i), 0});
         return v;
     }();
     return r;
@@ -141,6 +153,7 @@ bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f
     // In canonical terms bm tiles the contiguous dimension of D.
     const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
     if (I % v.bm || J % v.bn || p.K % v.bk) return false;
+    if (!miw::tiled_supports_layout(i, p) || !miw::tiled_grid_fits(i, p)) return false;
     if (!aligned16(p.A) || !aligned16(p.B) || !aligned16(p.D) || (p.use_c && !aligned16(p.C))) return false;
     if (p.lda % 8 || p.ldb % 8 || p.sa % 8 || p.sb % 8) return false;
     const long cper = 16 / (long)dtype_size(c_type), dper = 16 / (long)dtype_size(d_type);
@@ -163,7 +176,15 @@ int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc,
     const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
     int best = -1;
     long best_wgs = -1;
-    for (int i = 0; i < miw::tiled_variant_count(); i++) {
+    // Tiles from large to small; of two kernels for one tile the ping-pong form goes first.
+    std::vector<int> order;
+    for (int i = 0; i < miw::tiled_variant_count(); i++) order.push_back(i);
+    std::stable_sort(order.begin(), order.end(), [](int a, int b) {
+        const miw::tiled_variant &va = miw::tiled_variant_at(a), &vb = miw::tiled_variant_at(b);
+        if (va.bm * va.bn != vb.bm * vb.bn) return va.bm * va.bn > vb.bm * vb.bn;
+        return va.pingpong > vb.pingpong;
+    });
+    for (int i : order) {
         if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk)) continue;
         const miw::tiled_variant &v = miw::tiled_variant_at(i);
         const long wgs = (I / v.bm) * (J / v.bn) * p.batch;
@@ -178,7 +199,8 @@ int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc,
     return miw::tiled_variant_count() + 1;  // fragment-op kernel
 }
 
-int run_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, hipStream_t s)
+// Resolve the variant (0 = pick) and check that it can run this problem; touches no device.
+int check_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, int *variant_out)
 {
     const int nt = miw::tiled_variant_count();
     int variant = d->variant;
@@ -188,16 +210,25 @@ int run_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, hip
         if (f16acc && d->acc_chunk != 0 && d->acc_chunk != 16)
             return fail(MIW_ERR_UNSUPPORTED, "gemm: the fragment-op kernel rounds every 16 k-values (acc_chunk %d asked)",
                         d->acc_chunk);
-        HIP_TRY(miw::launch_gemm_fragops(p, d->c_type, d->d_type, f16acc, s));
-        return 0;
-    }
-    if (!tiled_fits(variant - 1, p, d->c_type, d->d_type, f16acc, d->acc_chunk))
+        if ((p.M / 16) * (p.N / 16) / 4 >= (1l << 31))
+            return fail(MIW_ERR_UNSUPPORTED, "gemm: %lld x %lld tiles of 16 x 16 do not fit the launch grid",
+                        (long long)(p.M / 16), (long long)(p.N / 16));
+    } else if (!tiled_fits(variant - 1, p, d->c_type, d->d_type, f16acc, d->acc_chunk)) {
         return fail(MIW_ERR_UNSUPPORTED,
                     "gemm: variant %d (%s) needs tile-divisible sizes, 16-byte aligned operands and leading "
-                    "dimensions%s",
+                    "dimensions, a tile count that fits the launch grid, and (ping-pong kernels) at most one operand "
+                    "with k contiguous%s",
                     variant, miw::tiled_variant_at(variant - 1).name,
                     f16acc ? ", alpha == 1, its own acc_chunk, and accumulators that fit in VGPRs" : "");
-    HIP_TRY(miw::launch_gemm_tiled(variant - 1, p, d->c_type, d->d_type, f16acc, s));
+    }
+    *variant_out = variant;
+    return 0;
+}
+
+int launch_gemm(int variant, const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, hipStream_t s)
+{
+    if (variant == miw::tiled_variant_count() + 1) HIP_TRY(miw::launch_gemm_fragops(p, d->c_type, d->d_type, f16acc, s));
+    else HIP_TRY(miw::launch_gemm_tiled(variant - 1, p, d->c_type, d->d_type, f16acc, s));
     return 0;
 }
 
@@ -218,6 +249,7 @@ int miw_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(MIW_ERR_UNSUPPORTED, "init: kernels are built for gfx950, device is %s", prop.gcnArchName);
     g_cu_count = prop.multiProcessorCount;
+    g_initialized.store(true, std::memory_order_release);
     g_err[0] = 0;
     return 0;
 }
@@ -225,6 +257,7 @@ int miw_init(int device)
 int miw_device_info_get(miw_device_info *out)
 {
     if (!out) return fail(MIW_ERR_NULL_POINTER, "device_info: null output");
+    REQUIRE_INIT("device_info");
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     hipDeviceProp_t prop;
@@ -250,6 +283,7 @@ int miw_malloc(void **out, size_t bytes)
     if (!out) return fail(MIW_ERR_NULL_POINTER, "malloc: null output");
     *out = nullptr;
     if (bytes == 0) return 0;
+    REQUIRE_INIT("malloc");
     HIP_TRY(hipMalloc(out, bytes));
     return 0;
 }
@@ -257,6 +291,7 @@ int miw_malloc(void **out, size_t bytes)
 int miw_free(void *p)
 {
     if (!p) return 0;
+    REQUIRE_INIT("free");
     HIP_TRY(hipFree(p));
     return 0;
 }
@@ -265,6 +300,7 @@ int miw_memcpy_h2d(void *dst, const void *src, size_t bytes)
 {
     if (bytes == 0) return 0;
     if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "memcpy_h2d: null pointer");
+    REQUIRE_INIT("memcpy_h2d");
     HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
     return 0;
 }
@@ -273,6 +309,7 @@ int miw_memcpy_d2h(void *dst, const void *src, size_t bytes)
 {
     if (bytes == 0) return 0;
     if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "memcpy_d2h: null pointer");
+    REQUIRE_INIT("memcpy_d2h");
     HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
     return 0;
 }
@@ -281,6 +318,7 @@ int miw_memcpy_d2d(void *dst, const void *src, size_t bytes)
 {
     if (bytes == 0) return 0;
     if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "memcpy_d2d: null pointer");
+    REQUIRE_INIT("memcpy_d2d");
     HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice));
     return 0;
 }
@@ -289,6 +327,7 @@ int miw_memset(void *dst, int byte, size_t bytes)
 {
     if (bytes == 0) return 0;
     if (!dst) return fail(MIW_ERR_NULL_POINTER, "memset: null pointer");
+    REQUIRE_INIT("memset");
     HIP_TRY(hipMemset(dst, byte, bytes));
     return 0;
 }
@@ -296,6 +335,7 @@ int miw_memset(void *dst, int byte, size_t bytes)
 int miw_stream_create(void **out)
 {
     if (!out) return fail(MIW_ERR_NULL_POINTER, "stream_create: null output");
+    REQUIRE_INIT("stream_create");
     hipStream_t s;
     HIP_TRY(hipStreamCreate(&s));  // default priority only
     *out = (void *)s;
@@ -311,6 +351,7 @@ int miw_stream_destroy(void *stream)
 
 int miw_sync(void *stream)
 {
+    REQUIRE_INIT("sync");
     if (stream) HIP_TRY(hipStreamSynchronize(as_stream(stream)));
     else HIP_TRY(hipDeviceSynchronize());
     return 0;
@@ -319,6 +360,7 @@ int miw_sync(void *stream)
 int miw_event_create(void **out)
 {
     if (!out) return fail(MIW_ERR_NULL_POINTER, "event_create: null output");
+    REQUIRE_INIT("event_create");
     hipEvent_t e;
     HIP_TRY(hipEventCreate(&e));
     *out = (void *)e;
@@ -335,6 +377,7 @@ int miw_event_destroy(void *event)
 int miw_event_record(void *event, void *stream)
 {
     if (!event) return fail(MIW_ERR_NULL_POINTER, "event_record: null event");
+    REQUIRE_INIT("event_record");
     HIP_TRY(hipEventRecord((hipEvent_t)event, as_stream(stream)));
     return 0;
 }
@@ -380,6 +423,7 @@ int miw_frag_load(int use, int dtype, int layout, int addr_space, int m, int n, 
     if (!addr || !frag) return fail(MIW_ERR_NULL_POINTER, "frag_load: null pointer");
     if (stride < 16) return fail(MIW_ERR_INVALID_VALUE, "frag_load: stride %lld smaller than the tile", (long long)stride);
     if ((uintptr_t)addr & (dtype_size(dtype) - 1)) return fail(MIW_ERR_MISALIGNED, "frag_load: misaligned address");
+    REQUIRE_INIT("frag_load");
     HIP_TRY(miw::launch_frag_load(use, dtype, layout == MIW_ROW_MAJOR, addr_space, addr, (long)stride, frag,
                                   as_stream(stream)));
     return 0;
@@ -395,6 +439,7 @@ int miw_frag_store(int dtype, int layout, int addr_space, int m, int n, int k, v
     if (!addr || !frag) return fail(MIW_ERR_NULL_POINTER, "frag_store: null pointer");
     if (stride < 16) return fail(MIW_ERR_INVALID_VALUE, "frag_store: stride %lld smaller than the tile", (long long)stride);
     if ((uintptr_t)addr & (dtype_size(dtype) - 1)) return fail(MIW_ERR_MISALIGNED, "frag_store: misaligned address");
+    REQUIRE_INIT("frag_store");
     HIP_TRY(miw::launch_frag_store(dtype, layout == MIW_ROW_MAJOR, addr_space, addr, frag, (long)stride,
                                    as_stream(stream)));
     return 0;
@@ -404,6 +449,7 @@ int miw_frag_fill(int dtype, float value, void *frag, void *stream)
 {
     if (!valid_dtype(dtype)) return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: %d", dtype);
     if (!frag) return fail(MIW_ERR_NULL_POINTER, "frag_fill: null pointer");
+    REQUIRE_INIT("frag_fill");
     HIP_TRY(miw::launch_frag_fill(dtype, value, frag, as_stream(stream)));
     return 0;
 }
@@ -413,6 +459,7 @@ int miw_frag_map(int dtype, int op, float scalar, const void *in, void *out, siz
     if (!valid_dtype(dtype)) return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: %d", dtype);
     if (op != MIW_OP_MUL && op != MIW_OP_ADD) return fail(MIW_ERR_INVALID_VALUE, "frag_map: unknown operator %d", op);
     if (n_elems && (!in || !out)) return fail(MIW_ERR_NULL_POINTER, "frag_map: null pointer");
+    REQUIRE_INIT("frag_map");
     HIP_TRY(miw::launch_frag_map(dtype, op, scalar, in, out, n_elems, as_stream(stream)));
     return 0;
 }
@@ -425,6 +472,7 @@ int miw_frag_mma(int a_layout, int b_layout, int c_type, int d_type, const void 
     if (!valid_dtype(c_type) || !valid_dtype(d_type))
         return fail(MIW_ERR_INVALID_TYPE, "Invalid element type for WMMA: c=%d d=%d", c_type, d_type);
     if (!a_frag || !b_frag || !c_frag || !d_frag) return fail(MIW_ERR_NULL_POINTER, "frag_mma: null pointer");
+    REQUIRE_INIT("frag_mma");
     HIP_TRY(miw::launch_frag_mma(c_type, d_type, a_frag, b_frag, c_frag, d_frag, as_stream(stream)));
     return 0;
 }
@@ -448,6 +496,7 @@ int miw_wmma_mac(const miw_mac_desc *d, const void *A, const void *B, const void
     if (((uintptr_t)A & 1) || ((uintptr_t)B & 1) || ((uintptr_t)D & (dtype_size(d->d_type) - 1)) ||
         (d->use_c && ((uintptr_t)C & (dtype_size(d->c_type) - 1))))
         return fail(MIW_ERR_MISALIGNED, "wmma_mac: operand pointer not aligned to its element type");
+    REQUIRE_INIT("wmma_mac");
     HIP_TRY(miw::launch_wmma_mac(d->c_type, d->d_type, A, B, C, D, lda, ldb, ldc, ldd, d->a_layout == MIW_ROW_MAJOR,
                                  d->b_layout == MIW_ROW_MAJOR, d->c_layout == MIW_ROW_MAJOR,
                                  d->d_layout == MIW_ROW_MAJOR, d->use_c != 0, d->addr_space == MIW_AS_SHARED, d->alpha,
@@ -477,6 +526,21 @@ int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out)
     out->block_m = v.bm; out->block_n = v.bn; out->block_k = v.bk;
     out->waves_m = v.wm; out->waves_n = v.wn; out->stages = v.stages; out->lds_bytes = v.lds_bytes;
     out->f16_accumulate = miw::tiled_supports_f16acc(variant - 1) ? 1 : 0;
+    out->pingpong = v.pingpong;
+    return 0;
+}
+
+int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *supported)
+{
+    if (!supported) return fail(MIW_ERR_NULL_POINTER, "gemm_variant_supports: null output");
+    const int nt = miw::tiled_variant_count();
+    if (variant < 1 || variant > nt + 1) return fail(MIW_ERR_INVALID_VALUE, "gemm_variant_supports: unknown variant %d", variant);
+    miw::gemm_params p;
+    bool f16acc;
+    static char dummy alignas(16);
+    if (int rc = resolve_gemm(desc, &dummy, &dummy, &dummy, &dummy, &p, &f16acc)) return rc;
+    if (variant == nt + 1) *supported = !(f16acc && desc->acc_chunk != 0 && desc->acc_chunk != 16);
+    else *supported = tiled_fits(variant - 1, p, desc->c_type, desc->d_type, f16acc, desc->acc_chunk) ? 1 : 0;
     return 0;
 }
 
@@ -506,32 +570,42 @@ int miw_gemm(const miw_gemm_desc *desc, const void *A, const void *B, const void
 {
     miw::gemm_params p;
     bool f16acc;
+    int variant = 0;
     if (int rc = resolve_gemm(desc, A, B, C, D, &p, &f16acc)) return rc;
-    return run_gemm(desc, p, f16acc, as_stream(stream));
+    if (int rc = check_gemm(desc, p, f16acc, &variant)) return rc;
+    REQUIRE_INIT("gemm");
+    return launch_gemm(variant, desc, p, f16acc, as_stream(stream));
 }
 
 int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream,
                    int warmup, int iters, float *ms_each)
 {
-    if (iters < 1 || warmup < 0 || !ms_each) return fail(MIW_ERR_INVALID_VALUE, "gemm_bench: bad warmup/iters/output");
+    if (iters < 1 || iters > 100000 || warmup < 0 || !ms_each)
+        return fail(MIW_ERR_INVALID_VALUE, "gemm_bench: bad warmup/iters/output (at most 100000 timed launches per call)");
     miw::gemm_params p;
     bool f16acc;
+    int variant = 0;
     if (int rc = resolve_gemm(desc, A, B, C, D, &p, &f16acc)) return rc;
+    if (int rc = check_gemm(desc, p, f16acc, &variant)) return rc;
+    REQUIRE_INIT("gemm_bench");
     hipStream_t s = as_stream(stream);
     for (int i = 0; i < warmup; i++)
-        if (int rc = run_gemm(desc, p, f16acc, s)) return rc;
-    std::vector<hipEvent_t> ev((size_t)iters + 1);
-    for (auto &e : ev) HIP_TRY(hipEventCreate(&e));
+        if (int rc = launch_gemm(variant, desc, p, f16acc, s)) return rc;
+    std::vector<hipEvent_t> ev((size_t)iters + 1, nullptr);
     int rc = 0;
-    hipError_t he = hipEventRecord(ev[0], s);
+    hipError_t he = hipSuccess;
+    for (auto &e : ev)
+        if (he == hipSuccess) he = hipEventCreate(&e);
+    if (he == hipSuccess) he = hipEventRecord(ev[0], s);
     for (int i = 0; i < iters && rc == 0 && he == hipSuccess; i++) {
-        rc = run_gemm(desc, p, f16acc, s);
+        rc = launch_gemm(variant, desc, p, f16acc, s);
         if (rc == 0) he = hipEventRecord(ev[(size_t)i + 1], s);
     }
     if (rc == 0 && he == hipSuccess) he = hipEventSynchronize(ev[(size_t)iters]);
     for (int i = 0; i < iters && rc == 0 && he == hipSuccess; i++)
         he = hipEventElapsedTime(&ms_each[i], ev[(size_t)i], ev[(size_t)i + 1]);
-    for (auto &e : ev) (void)hipEventDestroy(e);
+    for (auto &e : ev)
+        if (e) (void)hipEventDestroy(e);
     if (rc) return rc;
     if (he != hipSuccess) return hip_fail(he, "gemm_bench");
     return 0;
@@ -541,6 +615,7 @@ int miw_launch_overhead_probe(int iters, int threads, float *cpu_us, float *gpu_
 {
     if (!cpu_us || !gpu_us || iters < 1 || threads < 1 || threads > 1024)
         return fail(MIW_ERR_INVALID_VALUE, "launch_overhead_probe: bad arguments");
+    REQUIRE_INIT("launch_overhead_probe");
     float *buf = nullptr;
     HIP_TRY(hipMalloc((void **)&buf, 4));
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -568,7 +643,9 @@ int miw_launch_overhead_probe(int iters, int threads, float *cpu_us, float *gpu_
 
 int miw_mfma_power_probe(int iters, int random_operands, double *tflops, double *shader_mhz, void *stream)
 {
-    if (!tflops || !shader_mhz || iters < 1) return fail(MIW_ERR_INVALID_VALUE, "mfma_power_probe: bad arguments");
+    if (!tflops || !shader_mhz || iters < 1 || iters > 10000000)
+        return fail(MIW_ERR_INVALID_VALUE, "mfma_power_probe: bad arguments (iters in 1..10000000)");
+    REQUIRE_INIT("mfma_power_probe");
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     hipDeviceProp_t prop;
@@ -611,7 +688,9 @@ int miw_mfma_power_probe(int iters, int random_operands, double *tflops, double 
 
 int miw_mfma_peak_probe(int iters, double *tflops, void *stream)
 {
-    if (!tflops || iters < 1) return fail(MIW_ERR_INVALID_VALUE, "mfma_peak_probe: bad arguments");
+    if (!tflops || iters < 1 || iters > 10000000)
+        return fail(MIW_ERR_INVALID_VALUE, "mfma_peak_probe: bad arguments (iters in 1..10000000)");
+    REQUIRE_INIT("mfma_peak_probe");
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     hipDeviceProp_t prop;
@@ -644,6 +723,7 @@ int miw_copy_probe(void *dst, const void *src, size_t bytes, void *stream)
 {
     if (!dst || !src) return fail(MIW_ERR_NULL_POINTER, "copy_probe: null pointer");
     if (((uintptr_t)dst | (uintptr_t)src | bytes) & 15) return fail(MIW_ERR_MISALIGNED, "copy_probe: needs 16-byte multiples");
+    REQUIRE_INIT("copy_probe");
     HIP_TRY(miw::launch_copy(dst, src, bytes, as_stream(stream)));
     return 0;
 }
@@ -675,6 +755,7 @@ int miw_kernel_lookup(const char *name, void **kernel)
 int miw_kernel_attributes_get(void *kernel, miw_kernel_attributes *out)
 {
     if (!kernel || !out) return fail(MIW_ERR_NULL_POINTER, "kernel_attributes: null argument");
+    REQUIRE_INIT("kernel_attributes");
     hipFuncAttributes a;
     HIP_TRY(hipFuncGetAttributes(&a, kernel));
     out->num_regs = a.numRegs;
@@ -688,6 +769,7 @@ int miw_kernel_attributes_get(void *kernel, miw_kernel_attributes *out)
 int miw_kernel_occupancy(void *kernel, size_t dynamic_shmem, int *min_grid, int *block)
 {
     if (!kernel || !min_grid || !block) return fail(MIW_ERR_NULL_POINTER, "kernel_occupancy: null argument");
+    REQUIRE_INIT("kernel_occupancy");
     HIP_TRY(hipOccupancyMaxPotentialBlockSize(min_grid, block, kernel, dynamic_shmem, 0));
     return 0;
 }
@@ -698,9 +780,16 @@ int miw_launch(void *kernel, const unsigned grid[3], const unsigned block[3], un
     bool known = false;
     for (auto &k : registry()) known = known || (void *)k.fn == kernel;
     if (!known) return fail(MIW_ERR_NOT_FOUND, "launch: not a kernel of this library");
+    for (auto &k : registry())
+        if ((void *)k.fn == kernel && k.launchable == 0)
+            return fail(MIW_ERR_UNSUPPORTED,
+                        "launch: '%s' takes a private argument block, a fixed workgroup size and up to 160 KiB of dynamic "
+                        "LDS; it can be looked up and queried, and is launched through miw_gemm",
+                        k.name.c_str());
     const unsigned long threads = (unsigned long)block[0] * block[1] * block[2];
     if (threads == 0 || (unsigned long)grid[0] * grid[1] * grid[2] == 0)
         return fail(MIW_ERR_INVALID_VALUE, "launch: empty grid or block");
+    REQUIRE_INIT("launch");
     hipFuncAttributes a;
     HIP_TRY(hipFuncGetAttributes(&a, kernel));
     if (threads > (unsigned long)a.maxThreadsPerBlock)

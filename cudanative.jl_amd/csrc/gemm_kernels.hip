@@ -3,20 +3,24 @@
 // gemm_tile_*.hip translation units (one per tile family, so that they build in parallel).
 #include "gemm_tiled.hpp"
 
+#include <mutex>
+#include <unordered_map>
+
 namespace miw {
 
 // --------------------------------------------------------------- variants --
 
 static const tiled_variant g_variants[] = {
-    // name                    bm   bn  bk     wm wn slots lds
-    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2},
-    {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2},
-    {"tile256x128_w4x2", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2},
-    {"tile128x256_w2x4", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2},
-    {"tile128x128_w2x4_s4", 128, 128, KGRAN, 2, 4, 4, 4 * (128 + 128) * KGRAN * 2},
-    {"tile128x128_w2x2_s4", 128, 128, KGRAN, 2, 2, 4, 4 * (128 + 128) * KGRAN * 2},
-    {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2},
-    {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, 4, 4 * (64 + 64) * KGRAN * 2},
+    // name                    bm   bn  bk     wm wn slots lds (pingpong: ring depth of a K-major operand, largest ring)
+    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2, 0},
+    {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2, 0},
+    {"tile256x128_w4x2", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 0},
+    {"tile128x256_w2x4", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 0},
+    {"tile128x128_w2x4_s4", 128, 128, KGRAN, 2, 4, 4, 4 * (128 + 128) * KGRAN * 2, 0},
+    {"tile128x128_w2x2_s4", 128, 128, KGRAN, 2, 2, 4, 4 * (128 + 128) * KGRAN * 2, 0},
+    {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2, 0},
+    {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, 4, 4 * (64 + 64) * KGRAN * 2, 0},
+    {"tile256x256_pingpong", 256, 256, KGRAN, 2, 4, 3, 160 * 1024, 1},
 };
 
 int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }
@@ -25,6 +29,7 @@ int tiled_f16acc_chunk() { return KGRAN; }
 bool tiled_supports_f16acc(int i)
 {
     const tiled_variant &v = g_variants[i];
+    if (v.pingpong) return false;  // fp32 accumulation only
     return waves_per_simd(v.bm, v.bn, v.wm * v.wn * 64) >= 2;
 }
 
@@ -37,6 +42,8 @@ const void *tiled_kernel_128x128_w2x4_s4(bool xk, bool yk, int c_type, int d_typ
 const void *tiled_kernel_128x128_w2x2_s4(bool xk, bool yk, int c_type, int d_type, bool f16acc);
 const void *tiled_kernel_128x128_w2x2(bool xk, bool yk, int c_type, int d_type, bool f16acc);
 const void *tiled_kernel_64x64_w2x2(bool xk, bool yk, int c_type, int d_type, bool f16acc);
+const void *pp_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type);
+int pp_lds(int bm, int bn, bool xk, bool yk);
 
 // Tile shape in canonical (I, J) terms: bm applies to I, bn to J.
 static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, bool f16acc)
@@ -50,11 +57,49 @@ static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, 
         case 5: return tiled_kernel_128x128_w2x2_s4(xk, yk, c_type, d_type, f16acc);
         case 6: return tiled_kernel_128x128_w2x2(xk, yk, c_type, d_type, f16acc);
         case 7: return tiled_kernel_64x64_w2x2(xk, yk, c_type, d_type, f16acc);
+        case 8: return f16acc ? nullptr : pp_kernel(256, 256, xk, yk, c_type, d_type);
     }
     return nullptr;
 }
 
 const void *tiled_kernel_symbol(int i) { return pick_kernel(i, false, true, 1, 1, false); }
+
+// The workgroup index is a 32-bit grid coordinate and the kernels keep tile counts in int.
+bool tiled_grid_fits(int i, const gemm_params &g)
+{
+    const tiled_variant &v = g_variants[i];
+    const long I = g.d_row ? g.N : g.M, J = g.d_row ? g.M : g.N;
+    const long tiles = (I / v.bm) * (J / v.bn);
+    return tiles > 0 && tiles * (long)(v.wm * v.wn * 64) < (1l << 32) && tiles <= 0x7fffffffl;
+}
+
+// Which operands have k contiguous once the problem is in canonical form (see gemm_tiled.hpp).
+static void canonical_layout(const gemm_params &g, bool *xk, bool *yk)
+{
+    if (!g.d_row) { *xk = g.a_row != 0; *yk = g.b_row == 0; }
+    else { *xk = g.b_row == 0; *yk = g.a_row != 0; }
+}
+
+bool tiled_supports_layout(int i, const gemm_params &g)
+{
+    if (!g_variants[i].pingpong) return true;
+    bool xk, yk;
+    canonical_layout(g, &xk, &yk);
+    return pp_kernel(g_variants[i].bm, g_variants[i].bn, xk, yk, 1, 1) != nullptr;  // two K-major 256-row rings do not fit in LDS
+}
+
+// hipFuncAttributeMaxDynamicSharedMemorySize is a property of the kernel, not of the launch: set once.
+static hipError_t allow_dynamic_lds(const void *fn, int bytes)
+{
+    static std::mutex mu;
+    static std::unordered_map<const void *, int> done;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = done.find(fn);
+    if (it != done.end() && it->second >= bytes) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done[fn] = bytes;
+    return e;
+}
 
 hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type, bool f16acc, hipStream_t s)
 {
@@ -92,10 +137,11 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
 
     const void *fn = pick_kernel(i, xk, yk, c_type, d_type, f16acc);
     if (!fn) return hipErrorInvalidValue;
-    const int lds_bytes = v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    const int lds_bytes = v.pingpong ? pp_lds(v.bm, v.bn, xk, yk) : v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
+    hipError_t e = allow_dynamic_lds(fn, lds_bytes);
     if (e != hipSuccess) return e;
     void *args[] = {&p};
+    // the tile count fits: tiled_grid_fits() is part of the caller's check
     dim3 grid((unsigned)(p.tiles_i * p.tiles_j), (unsigned)g.batch);
     return hipLaunchKernel(fn, grid, dim3((unsigned)(v.wm * v.wn * 64)), args, (size_t)lds_bytes, s);
 }

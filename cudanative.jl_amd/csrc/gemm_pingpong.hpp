@@ -1,0 +1,452 @@
+// Ping-pong form of the LDS-tiled GEMM for gfx950 (fp32 accumulation): the two
+// wavefronts that share a SIMD take turns.  While one of them issues nothing
+// but the 32 MFMAs of a k-step (a "compute cluster", 512 cycles of matrix-core
+// time), the other one runs its "memory cluster": it reads its fragments of the
+// next k-step from LDS into registers and issues its share of the direct-to-LDS
+// loads that refill the ring.  A workgroup barrier ends every cluster and the
+// two swap roles.  The matrix cores never wait for an LDS read or for the issue
+// of a load (a wavefront alone on its SIMD loses 15-20 cycles of MFMA issue per
+// 1 KiB load it issues), and the two wavefronts never compete for them.
+//
+// Wavefronts 0-3 of the workgroup sit on SIMDs 0-3 and wavefronts 4-7 join
+// them in the same order; the second group enters the loop one barrier late, so
+// that it runs one cluster behind the first for the whole K loop.
+//
+// Same canonical problem, tile mapping and LDS chunk layouts as gemm_tiled.hpp
+// (P = X * Y, I contiguous in P).  What differs is how the ring is cut:
+//   I-major operand: four entries of 32 k-values (one k-step).  The loads of
+//       step t+3 are issued in the memory cluster of step t.
+//   K-major operand: three slots of 64 k-values (rows of 128 bytes, so that
+//       every direct-to-LDS load still fetches full 128-byte lines).  The loads
+//       of pair p+2 are issued in the two memory clusters of pair p, half each.
+// Either way a wavefront waits, at the end of memory cluster t, for the loads
+// it issued in cluster t-2 and earlier (s_waitcnt vmcnt(2 * loads per cluster)):
+// a load has two full clusters of both groups (about 2000 cycles) to land
+// before anyone waits for it, and the barriers between that wait and the first
+// read publish it to the other wavefronts.
+#pragma once
+#include "gemm_tiled.hpp"
+
+namespace miw {
+
+// Measurement switch, 0 in every shipped build: bit 0 drops the direct-to-LDS loads of the K loop,
+// bit 1 its fragment reads (the registers keep the prologue's fragments), bit 2 its MFMAs.  The
+// results are wrong; the timings say what each unit costs in cycles and, under the power cap, in clock.
+#ifndef MIW_PP_ABLATE
+#define MIW_PP_ABLATE 0
+#endif
+
+constexpr int PP_KMAJOR_SLOTS = 3;
+constexpr int PP_IMAJOR_ENTRIES = 4;
+
+constexpr int pp_operand_bytes(int rows, bool kmajor)
+{
+    return kmajor ? PP_KMAJOR_SLOTS * rows * KGRAN * 2 : PP_IMAJOR_ENTRIES * rows * BKS * 2;
+}
+constexpr int pp_lds_bytes(int bi, int bj, bool xk, bool yk) { return pp_operand_bytes(bi, xk) + pp_operand_bytes(bj, yk); }
+constexpr bool pp_fits(int bi, int bj, bool xk, bool yk) { return pp_lds_bytes(bi, bj, xk, yk) <= 160 * 1024; }
+
+// One operand of the ping-pong kernel: its ring in LDS, the loads that fill it
+// and the fragment reads.  R rows (or columns) of the tile, NT threads.
+template <int R, bool KMAJOR, int NT>
+struct pp_operand {
+    // loads per thread: per 64-k slot (K-major) or per 32-k entry (I-major)
+    static constexpr int NL = KMAJOR ? R * KGRAN / 8 / NT : R * BKS / 8 / NT;
+    // loads per thread and memory cluster
+    static constexpr int PER_CLUSTER = KMAJOR ? NL / 2 : NL;
+    static constexpr int UNIT_BYTES = KMAJOR ? R * KGRAN * 2 : R * BKS * 2;
+    static constexpr int UNITS = KMAJOR ? PP_KMAJOR_SLOTS : PP_IMAJOR_ENTRIES;
+    static constexpr int BYTES = UNITS * UNIT_BYTES;
+    static_assert(NL >= 1 && (!KMAJOR || NL % 2 == 0), "operand must divide over the workgroup");
+    static_assert(NT == 512, "lane offsets below assume 512 threads");
+
+    __device__ static inline unsigned lane_offset(int tid, int ld)
+    {
+        if constexpr (KMAJOR) {
+            return slot_loader<R, true, NT>::lane_offset(tid, ld);
+        } else {
+            // chunk tid of the entry: i-block tid / 256, k-row (tid / 8) % 32, chunk position tid % 8
+            const int k = (tid >> 3) & 31, cpos = tid & 7, iblk = tid >> 8;
+            const int c = cpos ^ (2 * i_major_swizzle(k));
+            return 2u * (unsigned)(k * ld + iblk * 64 + c * 8);
+        }
+    }
+    // Element offset of load i of a unit relative to load 0 (uniform).
+    __device__ static inline long load_delta(int i, long ld)
+    {
+        if constexpr (KMAJOR) return (long)i * (NT / 8) * ld;
+        else return (long)i * (NT / 256) * 64;
+    }
+    // Elements between consecutive units in global memory.
+    __device__ static inline long unit_step(long ld) { return KMAJOR ? (long)KGRAN : (long)BKS * ld; }
+
+    // Fragment reads.  K-major: the reader of gemm_tiled.hpp on a 64-k slot.
+    // I-major: the same transpose reads on an entry of 32 k-rows (i-blocks of
+    // 64 i are 4 KiB apart instead of 8).
+    frag_reader<R, true> kr;
+    int ibase[4];
+    __device__ inline void init(int wave_row0, int lane)
+    {
+        if constexpr (KMAJOR) {
+            kr.init(wave_row0, lane);
+        } else {
+            const int j = lane & 15, q = lane >> 4;
+            const int jq = j >> 2, jr = j & 3;
+            const int g = ((jq >> 1) & 1) | ((q & 1) << 1);
+            const int w16 = wave_row0 / 16;
+#pragma unroll
+            for (int m = 0; m < 4; m++)
+                ibase[m] = (w16 / 4) * 4096 + (8 * q + jq) * 128 + jr * 8 + ((((w16 & 3) + m) & 3) ^ g) * 32;
+        }
+    }
+    // Fragment T of k-step H (0/1: which half of the slot; ignored for I-major) out of the unit at `unit`.
+    template <int T, int H>
+    __device__ inline half8_t read(MIW_LDS const char *unit) const
+    {
+        if constexpr (KMAJOR) {
+            return kr.template read<T, H>(unit);
+        } else {
+            const int off = ibase[T & 3] + (T >> 2) * 4096;
+            fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(unit + off));
+            fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16((MIW_LDS fp16x4_t *)(unit + off + 512));
+            uint2_t l2 = __builtin_bit_cast(uint2_t, lo), h2 = __builtin_bit_cast(uint2_t, hi);
+            uint4_t v = {l2[0], l2[1], h2[0], h2[1]};
+            return __builtin_bit_cast(half8_t, v);
+        }
+    }
+};
+
+template <int BI, int BJ, int WI, int WJ, bool XK, bool YK, class CT, class DT>
+__global__ __launch_bounds__(WI *WJ * 64) __attribute__((amdgpu_waves_per_eu(2)))
+void k_gemm_pp(tiled_params p)
+{
+    constexpr int NT = WI * WJ * 64;
+    static_assert(NT == 512, "two wavefronts per SIMD");
+    constexpr int WTI = BI / WI, WTJ = BJ / WJ;
+    constexpr int TI = WTI / 16, TJ = WTJ / 16;
+    using xop = pp_operand<BI, XK, NT>;
+    using yop = pp_operand<BJ, YK, NT>;
+    constexpr int XB = xop::BYTES;
+    constexpr int ND = xop::PER_CLUSTER + yop::PER_CLUSTER;  // loads per thread and memory cluster
+    static_assert(pp_fits(BI, BJ, XK, YK), "ring does not fit in LDS");
+
+    extern __shared__ __attribute__((aligned(128))) char smem[];
+    MIW_LDS char *lds = (MIW_LDS char *)smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wi = wave % WI, wj = wave / WI;
+    const bool late_group = wave >= 4;
+
+    // Workgroup -> tile, as in k_gemm_tiled.
+    int tile_id;
+    {
+        const int total = p.tiles_i * p.tiles_j;
+        const int pid = blockIdx.x;
+        const int per = total >> 3, rem = total & 7;
+        const int xcd = pid & 7, loc = pid >> 3;
+        tile_id = xcd < rem ? xcd * (per + 1) + loc : rem * (per + 1) + (xcd - rem) * per + loc;
+    }
+    int ti0, tj0;
+    {
+        const int gsz = p.group_i * p.tiles_j;
+        const int gid = tile_id / gsz;
+        const int first = gid * p.group_i;
+        const int gi = min(p.tiles_i - first, p.group_i);
+        const int in = tile_id - gid * gsz;
+        ti0 = first + in % gi;
+        tj0 = in / gi;
+    }
+    const long bt = blockIdx.y;
+    const int i0 = ti0 * BI, j0 = tj0 * BJ;
+
+    const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
+    const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);
+    const unsigned xoff = xop::lane_offset(tid, (int)p.ldx);
+    const unsigned yoff = yop::lane_offset(tid, (int)p.ldy);
+
+    xop xr;
+    yop yr;
+    xr.init(wi * WTI, lane);
+    yr.init(wj * WTJ, lane);
+
+    const int q = lane >> 4, r = lane & 15;
+    const int row = i0 + wi * WTI + 4 * q;  // + 16*ti
+    const int col = j0 + wj * WTJ + r;      // + 16*tj
+    const CT *C = (const CT *)p.C + bt * p.sc;
+    DT *D = (DT *)p.D + bt * p.sd;
+
+    float4_t acc[TI][TJ];
+#pragma unroll
+    for (int a = 0; a < TI; a++)
+#pragma unroll
+        for (int b = 0; b < TJ; b++) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int NS = p.K / BKS;    // k-steps
+    const int NP = p.K / KGRAN;  // pairs of k-steps
+    const unsigned lds0 = (unsigned)(uintptr_t)lds;
+    const unsigned wave_dst = lds0 + (unsigned)wave * 1024u;
+
+    // ---- ring state (uniform).  I-major operand: the pair's two entries sit at `pair` and
+    // pair + UNIT_BYTES, pair toggling between 0 and 2 UNIT_BYTES.  K-major operand: `pair` is the
+    // slot of the current pair and `prev` the slot of the pair before it, which is the one being
+    // refilled (with pair pr + 2).
+    unsigned xpair = 0, xprev = 2 * xop::UNIT_BYTES, ypair = 0, yprev = 2 * yop::UNIT_BYTES;
+    int xnext = 0, ynext = 0;  // next unit to request (step index for I-major, pair index for K-major)
+    // Lane offsets of the loads of one unit: K-major loads differ by whole rows (a per-load lane
+    // offset keeps one uniform base address), I-major loads by 256 bytes (the instruction's offset field).
+    unsigned xvo[XK ? xop::NL : 1], yvo[YK ? yop::NL : 1];
+#pragma unroll
+    for (int i = 0; i < (XK ? xop::NL : 1); i++) xvo[i] = xoff + 2u * (unsigned)xop::load_delta(i, p.ldx);
+#pragma unroll
+    for (int i = 0; i < (YK ? yop::NL : 1); i++) yvo[i] = yoff + 2u * (unsigned)yop::load_delta(i, p.ldy);
+    // Load I of the unit at ring offset `unit` (bytes from the operand's region).
+    auto x_load = [&]<int I>(unsigned unit, std::integral_constant<int, I>) {
+        if constexpr (XK) lds_dma16_at<I * NT * 16, 0>(X, xvo[I], wave_dst + unit);
+        else lds_dma16_at<I * NT * 16, I * 256>(X, xvo[0], wave_dst + unit);
+    };
+    auto y_load = [&]<int I>(unsigned unit, std::integral_constant<int, I>) {
+        if constexpr (YK) lds_dma16_at<XB + I * NT * 16, 0>(Y, yvo[I], wave_dst + unit);
+        else lds_dma16_at<XB + I * NT * 16, I * 256>(Y, yvo[0], wave_dst + unit);
+    };
+    // Past the end of K the last unit is requested again, into a unit nobody reads any more.
+    auto x_advance = [&]() {
+        xnext++;
+        X += xnext < (XK ? NP : NS) ? xop::unit_step(p.ldx) : 0;
+    };
+    auto y_advance = [&]() {
+        ynext++;
+        Y += ynext < (YK ? NP : NS) ? yop::unit_step(p.ldy) : 0;
+    };
+    // Request number N (0 .. ND-1) of the memory cluster of k-step 2 pr + H: the X loads, then the Y loads.
+    auto cluster_request = [&]<int H, int N>(std::integral_constant<int, H>, std::integral_constant<int, N>) {
+        if constexpr (N < xop::PER_CLUSTER) {
+            if constexpr (XK) x_load(xprev, std::integral_constant<int, H * xop::NL / 2 + N>{});
+            else x_load(H == 0 ? (xpair ^ (2u * xop::UNIT_BYTES)) + xop::UNIT_BYTES : xpair, std::integral_constant<int, N>{});
+        } else {
+            constexpr int M = N - xop::PER_CLUSTER;
+            if constexpr (YK) y_load(yprev, std::integral_constant<int, H * yop::NL / 2 + M>{});
+            else y_load(H == 0 ? (ypair ^ (2u * yop::UNIT_BYTES)) + yop::UNIT_BYTES : ypair, std::integral_constant<int, M>{});
+        }
+    };
+    auto cluster_advance = [&]<int H>(std::integral_constant<int, H>) {
+        if constexpr (!XK || H == 1) x_advance();
+        if constexpr (!YK || H == 1) y_advance();
+    };
+    auto pair_advance = [&]() {
+        if constexpr (XK) {
+            xprev = xpair;
+            xpair = xpair + xop::UNIT_BYTES == xop::BYTES ? 0 : xpair + xop::UNIT_BYTES;
+        } else {
+            xpair ^= 2u * xop::UNIT_BYTES;
+        }
+        if constexpr (YK) {
+            yprev = ypair;
+            ypair = ypair + yop::UNIT_BYTES == yop::BYTES ? 0 : ypair + yop::UNIT_BYTES;
+        } else {
+            ypair ^= 2u * yop::UNIT_BYTES;
+        }
+    };
+
+    // Prologue: K-major operands request pairs 0 and 1, I-major operands steps 0, 1 and 2; everything
+    // lands and is published before the loop starts.
+#pragma unroll
+    for (int u = 0; u < (XK ? 2 : 3); u++) {
+        [&]<int... I>(std::integer_sequence<int, I...>) {
+            (x_load((unsigned)(u * xop::UNIT_BYTES), std::integral_constant<int, I>{}), ...);
+        }(std::make_integer_sequence<int, xop::NL>{});
+        x_advance();
+    }
+#pragma unroll
+    for (int u = 0; u < (YK ? 2 : 3); u++) {
+        [&]<int... I>(std::integer_sequence<int, I...>) {
+            (y_load((unsigned)(u * yop::UNIT_BYTES), std::integral_constant<int, I>{}), ...);
+        }(std::make_integer_sequence<int, yop::NL>{});
+        y_advance();
+    }
+    wait_loads_and_barrier<0>();
+
+    half8_t fx[TI], fy[TJ];
+    if constexpr (MIW_PP_ABLATE & 2) {
+        [&]<int... U>(std::integer_sequence<int, U...>) { ((fx[U] = xr.template read<U, 0>(lds)), ...); }(std::make_integer_sequence<int, TI>{});
+        [&]<int... U>(std::integer_sequence<int, U...>) { ((fy[U] = yr.template read<U, 0>(lds + XB)), ...); }(std::make_integer_sequence<int, TJ>{});
+    }
+    // Memory cluster of step 2 pr + H: the fragments of the step, with the cluster's requests
+    // issued at even distances between the reads (the reads are bound by the LDS, which the four
+    // wavefronts that are in their memory cluster share: a load issued between two of them costs
+    // no extra time).
+    constexpr int NFRAG = TI + TJ;
+    // Fragment unit U of a step (the TI x-fragments, then the TJ y-fragments), preceded by the
+    // requests that go out before it: request N before unit N * NFRAG / ND.
+    auto cluster_unit = [&]<int H, int U>(MIW_LDS const char *xu, MIW_LDS const char *yu, std::integral_constant<int, H> h,
+                                          std::integral_constant<int, U>) {
+        [&]<int... N>(std::integer_sequence<int, N...>) {
+            (([&] {
+                 if constexpr (N * NFRAG / ND == U && !(MIW_PP_ABLATE & 1)) {
+                     cluster_request(h, std::integral_constant<int, N>{});
+                     __builtin_amdgcn_sched_barrier(0);
+                 }
+             }()),
+             ...);
+        }(std::make_integer_sequence<int, ND>{});
+        if constexpr (MIW_PP_ABLATE & 2) {
+            asm volatile("" : "+v"(fx[U % TI]), "+v"(fy[U % TJ]));
+        } else {
+            if constexpr (U < TI) fx[U] = xr.template read<U, H>(xu);
+            else fy[U - TI] = yr.template read<U - TI, H>(yu);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto memory_cluster = [&]<int H>(std::integral_constant<int, H> h) {
+        MIW_LDS const char *xu = lds + xpair + (XK ? 0 : H * xop::UNIT_BYTES);
+        MIW_LDS const char *yu = lds + XB + ypair + (YK ? 0 : H * yop::UNIT_BYTES);
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            (cluster_unit(xu, yu, h, std::integral_constant<int, U>{}), ...);
+        }(std::make_integer_sequence<int, NFRAG>{});
+        cluster_advance(h);
+        if constexpr (H == 1) pair_advance();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto compute_cluster = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        // serpentine order: every MFMA changes exactly one of its two operand fragments
+#pragma unroll
+        for (int a = 0; a < TI; a++)
+#pragma unroll
+            for (int bb = 0; bb < TJ; bb++) {
+                const int b = serpentine_column(a * TJ + bb, TJ);
+                if constexpr (!(MIW_PP_ABLATE & 4)) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[a], fy[b], acc[a][b], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    };
+
+    // Folding C.  With alpha == 1 the C operand is added into the accumulators during the last
+    // NFOLD k-steps, CPT MFMA tiles per memory cluster, so that the memory system delivers C
+    // while the matrix cores run and the epilogue only stores.  The tiles of fold step S are
+    // requested at the end of the memory cluster with ordinary loads into registers (the lane
+    // fetches the 16 bytes it owns); they are the youngest loads of their cluster, so the wait at
+    // the end of the cluster two steps later covers them, and that cluster adds them in: C has
+    // two clusters of both wavefront groups to arrive.  Three register stages rotate.  Tiles go in
+    // the order of their addresses: 16 rows (64 bytes, the instruction's offset field) further
+    // down a column block, then the next 16 columns.  The accumulators are registers, so the
+    // folding steps are unrolled.
+    constexpr int CPT = 1;
+    constexpr int NTILE = TI * TJ;
+    constexpr int NFOLD = NTILE / CPT;
+    constexpr bool CAN_FOLD = __is_same(CT, float) && TI % CPT == 0 && NFOLD % 2 == 0;
+    bool fold_c = false;
+    // (the lane offset into the tile of C is kept in 32 bits)
+    if constexpr (CAN_FOLD) fold_c = p.use_c && !p.c_trans && p.alpha == 1.0f && NS >= NFOLD + 2 && p.ldc < (1l << 22);
+    float4_t cst[3][CPT];
+    const char *cnext = (const char *)(C + (long)j0 * p.ldc + i0);
+    const unsigned coff = 4u * (unsigned)((wj * WTJ + r) * (int)p.ldc + wi * WTI + 4 * q);
+    auto fold_request = [&]<int S>(std::integral_constant<int, S>) {
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            (([&] {
+                 constexpr int a = (S * CPT + U) % TI;
+                 asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(cst[S % 3][U]) : "v"(coff), "s"(cnext), "n"(64 * a) : "memory");
+                 if constexpr (a == TI - 1) cnext += 64 * p.ldc;
+             }()),
+             ...);
+        }(std::make_integer_sequence<int, CPT>{});
+    };
+    auto fold_add = [&]<int S>(std::integral_constant<int, S>) {
+#pragma unroll
+        for (int u = 0; u < CPT; u++) {
+            const int a = (S * CPT + u) % TI, b = (S * CPT + u) / TI;
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[a][b][e] = __builtin_fmaf(p.beta, cst[S % 3][u][e], acc[a][b][e]);
+        }
+    };
+    // One k-step: memory cluster, barrier, compute cluster, barrier.  FS >= 0: fold step FS.
+    auto step = [&]<int H, int FS>(std::integral_constant<int, H> h, std::integral_constant<int, FS>) {
+        memory_cluster(h);
+        if constexpr (FS >= 0) {
+            fold_request(std::integral_constant<int, FS>{});
+            __builtin_amdgcn_sched_barrier(0);
+            // fold step FS issues ND + CPT loads; steps before the first fold step issue ND
+            constexpr int YOUNGER = 2 * ND + (FS >= 1 ? 2 : 1) * CPT;
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt((YOUNGER & 15) | (7 << 4) | (0 << 8) | ((YOUNGER >> 4) << 14));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (FS >= 2) fold_add(std::integral_constant<int, FS - 2>{});
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            wait_loads_and_barrier<2 * ND>();
+        }
+        compute_cluster();
+        __builtin_amdgcn_s_barrier();
+    };
+    constexpr std::integral_constant<int, -1> no_fold{};
+
+    if (late_group) __builtin_amdgcn_s_barrier();
+    const int NPM = fold_c ? NP - NFOLD / 2 : NP;
+    for (int pr = 0; pr < NPM; pr++) {
+        step(std::integral_constant<int, 0>{}, no_fold);
+        step(std::integral_constant<int, 1>{}, no_fold);
+    }
+    if constexpr (CAN_FOLD) {
+        if (fold_c) {
+            [&]<int... G>(std::integer_sequence<int, G...>) {
+                ((step(std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * G>{}),
+                  step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2 * G + 1>{})),
+                 ...);
+            }(std::make_integer_sequence<int, NFOLD / 2>{});
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may outlive the workgroup's LDS
+    if constexpr (CAN_FOLD) {
+        if (fold_c) {
+            fold_add(std::integral_constant<int, NFOLD - 2>{});
+            fold_add(std::integral_constant<int, NFOLD - 1>{});
+        }
+    }
+    if (!late_group) __builtin_amdgcn_s_barrier();
+
+    // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
+    auto read_c = [&](int a, int b, bool trans) -> float4_t {
+        float4_t c;
+        const int ii = row + 16 * a, jj = col + 16 * b;
+        if (trans) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) c[v] = (float)C[(long)(ii + v) * p.ldc + jj];
+        } else if constexpr (__is_same(CT, float)) {
+            c = *(const float4_t *)(C + (long)jj * p.ldc + ii);
+        } else {
+            half4_t h = *(const half4_t *)(C + (long)jj * p.ldc + ii);
+            c = float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+        }
+        return c;
+    };
+    auto epilogue = [&](bool with_c, bool trans) {
+#pragma unroll
+        for (int b = 0; b < TJ; b++)
+#pragma unroll
+            for (int a = 0; a < TI; a++) {
+                float4_t v = acc[a][b];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] *= p.alpha;
+                if (with_c) {
+                    float4_t c = read_c(a, b, trans);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
+                }
+                DT *dst = D + (long)(col + 16 * b) * p.ldd + (row + 16 * a);
+                if constexpr (__is_same(DT, float)) {
+                    *(float4_t *)dst = v;
+                } else {
+                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    *(half4_t *)dst = h;
+                }
+            }
+    };
+    if (!p.use_c || fold_c) epilogue(false, false);
+    else if (p.c_trans) epilogue(true, true);
+    else epilogue(true, false);
+}
+
+}  // namespace miw

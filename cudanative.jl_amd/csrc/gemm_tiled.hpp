@@ -111,6 +111,20 @@ __device__ inline void lds_dma16_imm(const void *base, unsigned voff, unsigned l
                  : "memory", "m0");
 }
 
+// The same with both addresses given as a uniform base plus a compile-time byte offset: lane l
+// fetches base + G_IMM + voff[l] into LDS byte lds_base + DST_IMM + 16*l.  M0 is written by the
+// addition itself (the instruction's offset field advances the LDS address as well as the global
+// one, so M0 is set back by as much).
+template <int DST_IMM, int G_IMM>
+__device__ inline void lds_dma16_at(const void *base, unsigned voff, unsigned lds_base)
+{
+    static_assert(G_IMM >= 0 && G_IMM < 4096, "instruction offset field");
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4"
+                 :
+                 : "s"(lds_base), "v"(voff), "s"(base), "n"(DST_IMM - G_IMM), "n"(G_IMM)
+                 : "memory", "m0", "scc");
+}
+
 __device__ inline int i_major_swizzle(int k) { return ((k >> 1) & 1) | (((k >> 3) & 1) << 1); }
 
 // ------------------------------------------------------------ slot loader --
@@ -214,6 +228,12 @@ constexpr int dma_after_mfma(int m, int nmfma, int ndma)
         if (k * nmfma / (ndma < nmfma ? ndma : nmfma) == m) return k;
     return -1;
 }
+
+// MFMA number m of a step works on tile (m / tj, serpentine_column(m, tj)): rows of tiles are
+// walked alternately left to right and right to left, so that every MFMA changes exactly one of
+// its two operand fragments.  Under the power cap that is worth 7 % of matrix-core throughput on
+// random data against the row-by-row order, in which both operands change at the end of a row.
+constexpr int serpentine_column(int m, int tj) { return ((m / tj) & 1) ? tj - 1 - m % tj : m % tj; }
 
 template <int TI, int TJ>
 struct frag_set {

@@ -43,6 +43,7 @@ const char *frag_kernel_name(int i);
 struct tiled_variant {
     const char *name;
     int bm, bn, bk, wm, wn, stages, lds_bytes;
+    int pingpong;  // 1: the two wavefronts of a SIMD alternate between MFMA and memory clusters (gemm_pingpong.hpp)
 };
 int tiled_variant_count();
 const tiled_variant &tiled_variant_at(int i);
@@ -54,6 +55,10 @@ bool tiled_supports_f16acc(int i);
 // 16-byte alignment of pointers and leading dimensions, and (for fp16
 // accumulate) alpha == 1 and c_type == d_type == Float16.
 hipError_t launch_gemm_tiled(int i, const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s);
+// Does variant i have a kernel for this combination of operand layouts?
+bool tiled_supports_layout(int i, const gemm_params &p);
+// Does the problem's tile count fit the launch grid of variant i?
+bool tiled_grid_fits(int i, const gemm_params &p);
 const void *tiled_kernel_symbol(int i);
 
 hipError_t launch_mfma_peak(int blocks, int iters, float *sink, hipStream_t s);

@@ -61,8 +61,15 @@ def variants():
         _lib.check(lib.miw_gemm_variant_info_get(v, ctypes.byref(info)))
         out.append({"id": v, "name": info.name.decode(), "block": (info.block_m, info.block_n, info.block_k),
                     "waves": (info.waves_m, info.waves_n), "stages": info.stages, "lds_bytes": info.lds_bytes,
-                    "fragment_ops": bool(info.fragment_ops), "f16_accumulate": bool(info.f16_accumulate)})
+                    "fragment_ops": bool(info.fragment_ops), "f16_accumulate": bool(info.f16_accumulate), "pingpong": bool(info.pingpong)})
     return out
+
+
+def variant_supports(desc, variant):
+    """Can `variant` run this descriptor (operands assumed 16-byte aligned)?"""
+    ok = ctypes.c_int()
+    _lib.check(_lib.load().miw_gemm_variant_supports(ctypes.byref(desc), variant, ctypes.byref(ok)))
+    return bool(ok.value)
 
 
 def pick_variant(desc):

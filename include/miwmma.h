@@ -195,8 +195,13 @@ typedef struct miw_gemm_variant_info {
     int lds_bytes;
     int fragment_ops;   /* 1: built from load_a/load_b/mma on global memory, no LDS */
     int f16_accumulate; /* 1: has a Float16-accumulate form (accumulators fit in ordinary VGPRs) */
+    int pingpong;       /* 1: the two wavefronts of a SIMD alternate between matrix-core and memory phases;
+                           lds_bytes is then the largest ring over the operand layouts */
 } miw_gemm_variant_info;
 int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
+/* *supported = 1 when `variant` (1..count) can run this descriptor (tile divisibility, leading
+   dimensions, operand layouts, accumulate type; pointers are assumed 16-byte aligned), else 0. */
+int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *supported);
 /* Variant miw_gemm would pick for this descriptor. */
 int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant);
 /* acc_chunk miw_gemm would use for this descriptor (fp16 accumulate only). */

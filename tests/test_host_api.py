@@ -139,7 +139,7 @@ def test_struct_sizes_match_header(miw):
     L = miw._lib
     assert ctypes.sizeof(L.MacDesc) == 13 * 4 + 4 + 4 * 8      # 13 ints/floats, pad, 4 int64
     assert ctypes.sizeof(L.GemmDesc) == 7 * 8 + 11 * 4 + 4 + 5 * 8 + 8
-    assert ctypes.sizeof(L.GemmVariantInfo) == 64 + 9 * 4
+    assert ctypes.sizeof(L.GemmVariantInfo) == 64 + 10 * 4
     assert ctypes.sizeof(L.DeviceInfo) == 128 + 64 + 7 * 4 + 4 + 2 * 8 + 8
 
 
@@ -199,10 +199,17 @@ def test_variant_table_and_selection(miw):
     vs = G.variants()
     assert vs[-1]["fragment_ops"] and vs[-1]["name"] == "fragment_ops"
     assert all(v["lds_bytes"] <= 160 * 1024 for v in vs)
-    assert all(v["lds_bytes"] == v["stages"] * (v["block"][0] + v["block"][1]) * v["block"][2] * 2 for v in vs[:-1])
+    assert all(v["lds_bytes"] == v["stages"] * (v["block"][0] + v["block"][1]) * v["block"][2] * 2
+               for v in vs[:-1] if not v["pingpong"])
     by = {v["name"]: v["id"] for v in vs}
-    # 4096^3 fills 256 CUs with 256x256 tiles; small or odd shapes fall to smaller tiles / fragment ops
-    assert G.pick_variant(G.make_desc(4096, 4096, 4096)) == 1
+    # small or odd shapes fall to smaller tiles / fragment ops;
+    # 4096^3 fills 256 CUs with 256x256 tiles: the ping-pong kernel where its rings fit in LDS (at most one
+    # operand with k contiguous), else the kernel with two 64-k slots
+    W = miw.WMMA
+    assert vs[G.pick_variant(G.make_desc(4096, 4096, 4096)) - 1]["name"] == "tile256x256_pingpong"
+    rc = G.make_desc(4096, 4096, 4096, a_layout=W.RowMajor, b_layout=W.ColMajor)
+    assert G.pick_variant(rc) == 1 and not G.variant_supports(rc, by["tile256x256_pingpong"])
+    assert G.variant_supports(rc, 1) and not G.variant_supports(G.make_desc(128, 128, 128), 1)
     batched = vs[G.pick_variant(G.make_desc(128, 128, 128, batch=512)) - 1]
     assert batched["block"][:2] == (128, 128) and batched["stages"] == 2      # two workgroups per CU
     deep = vs[G.pick_variant(G.make_desc(2048, 2048, 2048)) - 1]
@@ -215,6 +222,8 @@ def test_variant_table_and_selection(miw):
     assert G.acc_chunk(d) == 16
     # fp16 accumulate rounds on the VALU: offered only where a lane's accumulators fit in 128 VGPRs
     for v in vs[:-1]:
+        if v["pingpong"]:
+            continue
         per_lane = v["block"][0] * v["block"][1] // (v["waves"][0] * v["waves"][1] * 64)
         assert v["f16_accumulate"] == (per_lane <= 128), v["name"]
     assert vs[-1]["f16_accumulate"]
@@ -236,3 +245,54 @@ def test_no_device_errors_are_clean(miw):
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
     assert out.returncode == 0, out.stderr
     assert out.stdout.strip() == "nodevice"
+
+
+def test_device_entries_need_init(miw):
+    """A fresh process that loads the library and skips miw_init: every entry that would touch the device
+    says so (after its argument checks), and the queries that need no device still answer."""
+    import subprocess, sys
+    code = ("import sys, ctypes; sys.path.insert(0, %r); from tests.conftest import load_package; m = load_package();\n"
+            "L = m._lib; lib = L.load(); p = ctypes.c_void_p(); N = L.ERR_NOT_INITIALIZED\n"
+            "assert lib.miw_malloc(ctypes.byref(p), 64) == N and b'miw_init' in lib.miw_last_error()\n"
+            "assert lib.miw_malloc(None, 64) == L.ERR_NULL_POINTER\n"
+            "assert lib.miw_free(ctypes.c_void_p(16)) == N and lib.miw_sync(None) == N\n"
+            "d = m.GEMM.make_desc(64, 64, 64); q = ctypes.c_void_p(4096)\n"
+            "assert lib.miw_gemm(ctypes.byref(d), q, q, q, q, None) == N\n"
+            "assert lib.miw_gemm(ctypes.byref(d), q, None, q, q, None) == L.ERR_NULL_POINTER\n"
+            "info = L.DeviceInfo(); assert lib.miw_device_info_get(ctypes.byref(info)) == N\n"
+            "k = ctypes.c_void_p(); assert lib.miw_kernel_lookup(b'wmma_mac_f32_f32', ctypes.byref(k)) == 0\n"
+            "u3 = (ctypes.c_uint * 3)\n"
+            "assert lib.miw_launch(k, u3(1, 1, 1), u3(64, 1, 1), 0, None, None) == N\n"
+            "assert m.GEMM.pick_variant(d) >= 1 and lib.miw_gemm_variant_count() >= 9\n"
+            "print('ok')\n") % ROOT
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", out.stderr
+
+
+def test_tiled_gemm_kernels_are_not_launchable_by_name(miw):
+    """The LDS-tiled kernels take a private argument block, a fixed workgroup and dynamic LDS: they can be
+    looked up (attribute queries) but miw_launch refuses them and points to miw_gemm."""
+    L = miw._lib
+    lib = L.load()
+    u3 = (ctypes.c_uint * 3)
+    for name in ("gemm_tile256x256_w2x4", "gemm_tile128x128_w2x2", "gemm_tile256x256_pingpong"):
+        k = ctypes.c_void_p()
+        assert lib.miw_kernel_lookup(name.encode(), ctypes.byref(k)) == 0 and k.value
+        assert lib.miw_launch(k, u3(1, 1, 1), u3(64, 1, 1), 0, None, None) == L.ERR_UNSUPPORTED
+        assert b"miw_gemm" in lib.miw_last_error()
+
+
+def test_tile_counts_that_overflow_the_grid_are_refused(miw):
+    L = miw._lib
+    lib = L.load()
+    q = ctypes.c_void_p(4096)
+    G = miw.GEMM
+    big = 1 << 30
+    for variant in (0, 1, 8, lib.miw_gemm_variant_count()):
+        d = G.make_desc(big, big, 64, variant=variant)
+        assert lib.miw_gemm(ctypes.byref(d), q, q, q, q, None) == L.ERR_UNSUPPORTED, variant
+    assert not G.variant_supports(G.make_desc(big, big, 64), 8)
+    # a launch holds fewer than 2^32 threads: 2^19 x 2^18 is 2^25 tiles of 64 x 64 with 256 threads each
+    # (too many) and 2^21 tiles of 256 x 256 with 512 (fine)
+    d = G.make_desc(1 << 19, 1 << 18, 64)
+    assert not G.variant_supports(d, 8) and G.variant_supports(d, 1)

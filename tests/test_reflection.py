@@ -52,6 +52,22 @@ def test_default_gemm_kernel_codegen_and_resources(miw):
     assert "ds_read_b64_tr_b16" not in _ops(next(iter(kk.values())))
 
 
+def test_auto_picked_4096_kernels_have_no_spills(miw):
+    """The kernels miw_gemm picks by itself for a 4096^3 problem, one per operand layout: the ping-pong
+    kernel where it exists (at most one operand with k contiguous), the two-slot kernel for two
+    K-major operands.  None of them may touch scratch memory, and all fit two wavefronts per SIMD."""
+    res = miw.reflection.kernel_resources()
+    picked = ["k_gemm_pp<256, 256, 2, 4, %s, float, float>" % l for l in ("true, false", "false, true", "false, false")]
+    picked.append("k_gemm_tiled<256, 256, 2, 4, 2, true, true, float, float, false>")
+    for name in picked:
+        (r,) = [v for k, v in res.items() if name in k]
+        assert r["spills"] == 0 and r["scratch"] == 0 and r["vgpr"] + r["agpr"] <= 256 and r["max_threads"] == 512, name
+    ops = _ops(next(iter(miw.reflection.code_gcn(picked[1]).values())))       # column-major A and B
+    assert ops["v_mfma_f32_16x16x32_f16"] >= 64 and ops["global_load_lds_dwordx4"] >= 8
+    assert ops["ds_read_b64_tr_b16"] >= 16 and ops["ds_read_b128"] >= 4
+    assert not any(o.startswith(("scratch_", "flat_", "ds_write", "v_accvgpr")) for o in ops)
+
+
 def test_tiled_kernels_keep_spills_out_of_the_steady_state(miw):
     """The rolled K loop (the two pipeline steps up to the backward branch) never touches scratch
     memory; the unrolled trips that fold C in may hold a few spills in one operand layout."""
