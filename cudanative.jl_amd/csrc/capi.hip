@@ -577,6 +577,132 @@ int miw_gemm(const miw_gemm_desc *desc, const void *A, const void *B, const void
     return launch_gemm(variant, desc, p, f16acc, as_stream(stream));
 }
 
+// ---- split-K ----
+
+}  // extern "C"
+
+namespace {
+
+struct splitk_plan {
+    miw::gemm_params full;   // the caller's problem
+    miw::gemm_params slice;  // first pass: `splits` independent products of K / splits k-values each
+    int variant;             // tiled variant of the first pass (1-based)
+    int splits;
+    size_t bytes;            // workspace the first pass fills
+};
+
+// The first pass of a split-K GEMM as a strided-batched problem over the K slices.
+miw::gemm_params splitk_slices(const miw::gemm_params &p, int splits, void *ws)
+{
+    miw::gemm_params q = p;
+    const long klen = p.K / splits;
+    q.K = klen;
+    q.C = nullptr; q.use_c = 0; q.alpha = 1.0f; q.beta = 0.0f;
+    q.D = ws;
+    q.c_row = q.d_row = p.d_row;
+    q.ldc = q.ldd = p.d_row ? p.N : p.M;
+    q.sc = q.sd = p.M * p.N;
+    q.sa = klen * (p.a_row ? 1 : p.lda);
+    q.sb = klen * (p.b_row ? p.ldb : 1);
+    q.batch = splits;
+    return q;
+}
+
+int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void *C, void *D, int splits, splitk_plan *out)
+{
+    bool f16acc;
+    miw::gemm_params p;
+    if (int rc = resolve_gemm(d, A, B, C, D, &p, &f16acc)) return rc;
+    if (f16acc) return fail(MIW_ERR_UNSUPPORTED, "gemm_splitk: Float32 accumulation only (slices are added in Float32)");
+    if (p.batch != 1) return fail(MIW_ERR_UNSUPPORTED, "gemm_splitk: one problem per call (batch %lld asked)", (long long)p.batch);
+    if (d->variant != 0) return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: the variant is chosen per slice; desc.variant must be 0");
+    if (splits < 0 || splits > 256) return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: splits must be 0 (choose) or 1..256, got %d", splits);
+    const int nt = miw::tiled_variant_count();
+    const int cus = g_cu_count > 0 ? g_cu_count : 256;
+    static char dummy alignas(16);
+    auto try_splits = [&](int s, int *variant, long *wgs) {
+        if (p.K % (64l * s)) return false;
+        const miw::gemm_params q = splitk_slices(p, s, &dummy);
+        const int v = pick_variant(q, MIW_F32, MIW_F32, false, 0);
+        if (v == nt + 1) return false;
+        const miw::tiled_variant &tv = miw::tiled_variant_at(v - 1);
+        const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
+        *variant = v;
+        *wgs = (I / tv.bm) * (J / tv.bn) * s;
+        return true;
+    };
+    int variant = 0;
+    long wgs = 0;
+    if (splits == 0) {
+        // Fewest slices that give every CU a workgroup: first with tiles of at least 128 x 128 and up
+        // to 16 slices of four LDS slots' worth of K or more (large tiles move less data per flop
+        // than a small tile saves in workspace traffic), else with any tile and up to 64 slices.
+        int best = 0;
+        for (int pass = 0; pass < 2 && (best == 0 || wgs < cus); pass++)
+            for (int s = 1; s <= (pass ? 64 : 16) && p.K / s >= (pass ? 128 : 256); s++) {
+                int v;
+                long w;
+                if (!try_splits(s, &v, &w)) continue;
+                const miw::tiled_variant &tv = miw::tiled_variant_at(v - 1);
+                if (pass == 0 && (w < cus || tv.bm * tv.bn < 128 * 128)) continue;
+                best = s; variant = v; wgs = w;
+                if (w >= cus) break;
+            }
+        splits = best;
+    } else if (!try_splits(splits, &variant, &wgs)) {
+        splits = 0;
+    }
+    if (splits == 0)
+        return fail(MIW_ERR_UNSUPPORTED,
+                    "gemm_splitk: needs K divisible by 64 * splits, M and N divisible by an LDS tile (64 at least), "
+                    "16-byte aligned operands and leading dimensions");
+    out->full = p;
+    out->splits = splits;
+    out->variant = variant;
+    out->bytes = (size_t)splits * (size_t)p.M * (size_t)p.N * sizeof(float);
+    out->slice = splitk_slices(p, splits, nullptr);
+    return 0;
+}
+
+int run_splitk(const miw_gemm_desc *d, splitk_plan &plan, void *ws, hipStream_t s)
+{
+    plan.slice.D = ws;
+    // the slices are checked against the real operand pointers (plan_splitk assumed aligned ones)
+    if (!tiled_fits(plan.variant - 1, plan.slice, MIW_F32, MIW_F32, false, 0))
+        return fail(MIW_ERR_MISALIGNED, "gemm_splitk: operands and workspace must be 16-byte aligned");
+    HIP_TRY(miw::launch_gemm_tiled(plan.variant - 1, plan.slice, MIW_F32, MIW_F32, false, s));
+    HIP_TRY(miw::launch_splitk_reduce(plan.full, d->c_type, d->d_type, plan.splits, (const float *)ws, s));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int miw_gemm_splitk_workspace(const miw_gemm_desc *desc, int splits, int *splits_out, size_t *bytes)
+{
+    if (!bytes) return fail(MIW_ERR_NULL_POINTER, "gemm_splitk_workspace: null output");
+    static char dummy alignas(16);
+    splitk_plan plan;
+    if (int rc = plan_splitk(desc, &dummy, &dummy, &dummy, &dummy, splits, &plan)) return rc;
+    if (splits_out) *splits_out = plan.splits;
+    *bytes = plan.bytes;
+    return 0;
+}
+
+int miw_gemm_splitk(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
+                    void *workspace, size_t workspace_bytes, void *stream)
+{
+    splitk_plan plan;
+    if (int rc = plan_splitk(desc, A, B, C, D, splits, &plan)) return rc;
+    if (!workspace) return fail(MIW_ERR_NULL_POINTER, "gemm_splitk: null workspace");
+    if (workspace_bytes < plan.bytes)
+        return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: workspace of %zu bytes, %d slices need %zu", workspace_bytes,
+                    plan.splits, plan.bytes);
+    REQUIRE_INIT("gemm_splitk");
+    return run_splitk(desc, plan, workspace, as_stream(stream));
+}
+
 int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream,
                    int warmup, int iters, float *ms_each)
 {

@@ -146,6 +146,55 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
     return hipLaunchKernel(fn, grid, dim3((unsigned)(v.wm * v.wn * 64)), args, (size_t)lds_bytes, s);
 }
 
+// ---------------------------------------------------------- split-K ---------
+
+// Second pass of the split-K GEMM.  The first pass left `splits` Float32 partial products in
+// `ws`, each I x J with I contiguous (canonical form: I runs along D's contiguous dimension);
+// this adds them in slice order and applies the scalars: D = alpha * sum_s P_s + beta * C.
+// One lane owns four consecutive i of one j.
+template <class CT, class DT>
+__global__ __launch_bounds__(256) void k_splitk_reduce(const float *ws, int splits, long I, long J, const CT *C, DT *D,
+                                                       long ldc, long ldd, int use_c, int c_trans, float alpha, float beta)
+{
+    const long quads = I / 4;
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= quads * J) return;
+    const long j = idx / quads, i = (idx - j * quads) * 4;
+    const float *src = ws + j * I + i;
+    float4_t sum = *(const float4_t *)src;
+    for (int s = 1; s < splits; s++) {
+        const float4_t v = *(const float4_t *)(src + (long)s * I * J);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum[e] += v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float v = alpha * sum[e];
+        if (use_c) {
+            const float c = (float)(c_trans ? C[(i + e) * ldc + j] : C[j * ldc + i + e]);
+            v = __builtin_fmaf(beta, c, v);
+        }
+        D[j * ldd + i + e] = (DT)v;
+    }
+}
+
+hipError_t launch_splitk_reduce(const gemm_params &g, int c_type, int d_type, int splits, const float *ws, hipStream_t s)
+{
+    const long I = g.d_row ? g.N : g.M, J = g.d_row ? g.M : g.N;
+    const int c_trans = g.d_row ? g.c_row == 0 : g.c_row != 0;
+    const long lanes = I / 4 * J;
+    const dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
+#define MIW_REDUCE(CT, DT)                                                                                          \
+    hipLaunchKernelGGL((k_splitk_reduce<CT, DT>), grid, block, 0, s, ws, splits, I, J, (const CT *)g.C, (DT *)g.D, \
+                       g.ldc, g.ldd, g.use_c, c_trans, g.alpha, g.beta)
+    if (c_type == 0 && d_type == 0) MIW_REDUCE(half_t, half_t);
+    else if (c_type == 0) MIW_REDUCE(half_t, float);
+    else if (d_type == 0) MIW_REDUCE(float, half_t);
+    else MIW_REDUCE(float, float);
+#undef MIW_REDUCE
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------ probes -------
 
 // Register-resident MFMA chain: 8 independent accumulators per wavefront.

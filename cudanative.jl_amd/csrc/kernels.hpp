@@ -60,6 +60,9 @@ bool tiled_supports_layout(int i, const gemm_params &p);
 // Does the problem's tile count fit the launch grid of variant i?
 bool tiled_grid_fits(int i, const gemm_params &p);
 const void *tiled_kernel_symbol(int i);
+// Second pass of the split-K GEMM: D = alpha * (sum over `splits` Float32 partial products in ws,
+// each M x N laid out as D without padding) + beta * C.
+hipError_t launch_splitk_reduce(const gemm_params &p, int c_type, int d_type, int splits, const float *ws, hipStream_t s);
 
 hipError_t launch_mfma_peak(int blocks, int iters, float *sink, hipStream_t s);
 // One 8-wavefront workgroup per block: 64 MFMAs per wavefront and iteration; ticks[2b], ticks[2b+1]:

@@ -22,6 +22,11 @@ def _dtype_code(T):
     return _lib.F16 if np.dtype(T) == np.float16 else _lib.F32
 
 
+def _stream(stream):
+    """A Stream object or a raw hipStream_t (None: the default stream) as the C ABI takes it."""
+    return getattr(stream, "handle", stream)
+
+
 def _ptr(x):
     if x is None:
         return None
@@ -42,13 +47,31 @@ def make_desc(M, N, K, *, a_layout=ColMajor, b_layout=ColMajor, c_layout=ColMajo
 
 def gemm(A, B, C, D, desc, stream=None):
     """Launch D = alpha*A*B + beta*C (asynchronous).  A, B, C, D: DeviceArray or raw device address."""
-    _lib.check(_lib.load().miw_gemm(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), stream))
+    _lib.check(_lib.load().miw_gemm(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), _stream(stream)))
+
+
+def splitk_workspace(desc, splits=0):
+    """(slices, workspace bytes) gemm_splitk would use for this descriptor (splits = 0: chosen by the library)."""
+    n, b = ctypes.c_int(), ctypes.c_size_t()
+    _lib.check(_lib.load().miw_gemm_splitk_workspace(ctypes.byref(desc), splits, ctypes.byref(n), ctypes.byref(b)))
+    return n.value, b.value
+
+
+def gemm_splitk(A, B, C, D, desc, splits=0, workspace=None, stream=None):
+    """Split-K launch of D = alpha*A*B + beta*C: K cut into slices whose Float32 products go through
+    `workspace` (a DeviceArray; allocated here when None) and are added in order by a second kernel."""
+    n, nbytes = splitk_workspace(desc, splits)
+    if workspace is None:
+        workspace = DeviceArray.undef(np.float32, nbytes // 4)
+    _lib.check(_lib.load().miw_gemm_splitk(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), n, _ptr(workspace),
+                                           workspace.nbytes, _stream(stream)))
+    return workspace
 
 
 def gemm_bench(A, B, C, D, desc, warmup=5, iters=20, stream=None):
     """Per-launch durations in milliseconds, HIP events on the launch stream."""
     ms = (ctypes.c_float * iters)()
-    _lib.check(_lib.load().miw_gemm_bench(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), stream,
+    _lib.check(_lib.load().miw_gemm_bench(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), _stream(stream),
                                           warmup, iters, ms))
     return np.array(ms[:], dtype=np.float64)
 

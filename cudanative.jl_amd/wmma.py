@@ -498,4 +498,4 @@ def mac(a_dev, b_dev, c_dev, d_dev, *, a_layout=ColMajor, b_layout=ColMajor, c_l
                         _layout_code(d_layout), _dtype_code(c_dtype), _dtype_code(d_dev.dtype), 1 if do_mac else 0,
                         addrspace, float(alpha), float(beta), lda, ldb, ldc, ldd)
     _lib.check(_lib.load().miw_wmma_mac(ctypes.byref(desc), a_dev.ptr, b_dev.ptr,
-                                        c_dev.ptr if c_dev is not None else None, d_dev.ptr, stream))
+                                        c_dev.ptr if c_dev is not None else None, d_dev.ptr, getattr(stream, "handle", stream)))

@@ -207,6 +207,19 @@ int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant);
 /* acc_chunk miw_gemm would use for this descriptor (fp16 accumulate only). */
 int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk);
 
+/* Split-K form of miw_gemm for problems with few output tiles and a long K: the chain of mma
+   calls over K (docs/src/device/wmma.md:51-52) is cut into `splits` equal slices (each a multiple
+   of 64 k-values), the LDS-tiled kernels write every slice's product as Float32 into `workspace`
+   (splits * m * n * 4 bytes, 16-byte aligned, contents on entry irrelevant), and a second kernel
+   adds the slices in order: D = alpha * sum_s A_s*B_s + beta*C.  The result does not depend on
+   timing; it differs from miw_gemm's by the rounding of one Float32 sum per slice.  Float32
+   accumulation, batch 1, desc.variant 0, M and N divisible by an LDS tile.  splits = 0 chooses
+   the fewest slices that give every CU a workgroup.  miw_gemm_splitk_workspace reports the slice
+   count and the bytes miw_gemm_splitk will ask for. */
+int miw_gemm_splitk_workspace(const miw_gemm_desc *desc, int splits, int *splits_out, size_t *bytes);
+int miw_gemm_splitk(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
 /* warmup untimed launches, then iters launches each bracketed by HIP events on
    `stream`; ms_each[i] receives launch i's duration in milliseconds. */
 int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D,

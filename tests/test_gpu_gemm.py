@@ -474,3 +474,94 @@ def test_bench_entry_reports_positive_times(gpu, orc):
     zero_tf, zero_mhz = gpu.mfma_power_probe(4000, random_operands=False)
     rand_tf, rand_mhz = gpu.mfma_power_probe(4000, random_operands=True)
     assert 100 < rand_tf <= zero_tf * 1.05 and 500 < rand_mhz <= zero_mhz * 1.05 < 2700    # random data never runs faster
+
+
+# ------------------------------------------------------------- split-K ------------
+
+def _run_splitk(gpu, orc, g, A, B, C, splits=0, prefill=None, static=False):
+    g = g.resolved()
+    dA, dB = gpu.DeviceArray(A), gpu.DeviceArray(B)
+    dC = gpu.DeviceArray(C) if C is not None else None
+    dt = orc.np_dtype(g.d_type)
+    dD = gpu.DeviceArray(np.full(g.stride_d, np.nan if prefill is None else prefill, dtype=dt))
+    desc = gpu.GEMM.make_desc(g.M, g.N, g.K, a_layout=_W(gpu, g.a_layout), b_layout=_W(gpu, g.b_layout),
+                              c_layout=_W(gpu, g.c_layout), d_layout=_W(gpu, g.d_layout),
+                              c_type=orc.np_dtype(g.c_type), d_type=dt, alpha=g.alpha, beta=g.beta,
+                              use_c=bool(g.use_c), lda=g.lda, ldb=g.ldb, ldc=g.ldc, ldd=g.ldd)
+    if static:
+        gpu.GEMM.gemm_splitk_static(dA, dB, dC, dD, desc, splits)
+    else:
+        gpu.GEMM.gemm_splitk(dA, dB, dC, dD, desc, splits)
+    gpu.synchronize()
+    return dD.to_host()
+
+
+@pytest.mark.parametrize("al,bl,cl,dl", itertools.product((0, 1), repeat=4))
+def test_splitk_exact_on_integer_inputs(gpu, orc, al, bl, cl, dl):
+    """Small integers: every slice's product and their sum are exact, so the split-K result must equal
+    the oracle bit for bit in every layout combination, for a forced and for a chosen slice count."""
+    g = orc.GemmDesc(M=256, N=128, K=1024, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, beta=-2.0)
+    A, B, C = _inputs(orc, g, 600 + al + 2 * bl + 4 * cl + 8 * dl, ints=True)
+    ref = orc.gemm(g, A, B, C)
+    for splits in (0, 1, 4, 16):
+        assert np.array_equal(_run_splitk(gpu, orc, g, A, B, C, splits), ref), (al, bl, cl, dl, splits)
+
+
+def test_splitk_random_types_scalars_and_padding(gpu, orc):
+    for ct, dt in itertools.product((0, 1), repeat=2):
+        g = orc.GemmDesc(M=192, N=320, K=2048, lda=200, ldb=2056, ldc=196, ldd=208, c_type=ct, d_type=dt,
+                         alpha=0.75, beta=-1.25)
+        A, B, C = _inputs(orc, g, 650 + 2 * ct + dt)
+        D = _run_splitk(gpu, orc, g, A, B, C, 8, prefill=3.0)
+        err = orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C))
+        assert err <= (TIGHT_F32 if dt == orc.F32 else 6e-4), (ct, dt, err)
+        assert np.count_nonzero(D == 3.0) >= (208 - 192) * 320          # padding between columns untouched
+    g = orc.GemmDesc(M=128, N=128, K=4096, use_c=0)
+    A, B, _ = _inputs(orc, g, 660)
+    D = _run_splitk(gpu, orc, g, A, B, None)
+    assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, None)) <= TIGHT_F32
+
+
+def test_splitk_slice_choice_and_errors(gpu, orc):
+    G = gpu.GEMM
+    L = gpu._lib
+    cus = gpu.device_info()["cu_count"]
+    n, nbytes = G.splitk_workspace(G.make_desc(512, 512, 16384))
+    assert n >= 2 and nbytes == n * 512 * 512 * 4 and 16384 % (64 * n) == 0
+    # enough workgroups for every CU: 256 x 256 tiles give 4, 64 x 64 tiles 64 per slice
+    assert n * 64 >= cus
+    assert G.splitk_workspace(G.make_desc(4096, 4096, 4096))[0] == 1          # already fills the chip
+    assert G.splitk_workspace(G.make_desc(512, 512, 16384), 32) == (32, 32 * 512 * 512 * 4)
+    for desc, splits, code in ((G.make_desc(512, 512, 1000 * 16), 3, L.ERR_UNSUPPORTED),     # K not divisible by 64 * 3
+                               (G.make_desc(48, 48, 1024), 2, L.ERR_UNSUPPORTED),            # no LDS tile divides 48
+                               (G.make_desc(128, 128, 1024, batch=2), 2, L.ERR_UNSUPPORTED),
+                               (G.make_desc(128, 128, 1024, variant=8), 2, L.ERR_INVALID_VALUE),
+                               (G.make_desc(128, 128, 1024), 300, L.ERR_INVALID_VALUE),
+                               (G.make_desc(128, 128, 1024, c_type=F16, d_type=F16, acc_type=F16), 2, L.ERR_UNSUPPORTED)):
+        with pytest.raises(gpu.MIWError) as e:
+            G.splitk_workspace(desc, splits)
+        assert e.value.code == code, (splits, e.value)
+    # a workspace that is too small is refused before anything is launched
+    g = orc.GemmDesc(M=128, N=128, K=1024)
+    A, B, C = _inputs(orc, g, 670)
+    dA, dB, dC, dD = (gpu.DeviceArray(x) for x in (A, B, C, np.zeros_like(C)))
+    small = gpu.DeviceArray.undef(np.float32, 128 * 128)
+    with pytest.raises(gpu.MIWError) as e:
+        G.gemm_splitk(dA, dB, dC, dD, G.make_desc(128, 128, 1024), 4, workspace=small)
+    assert e.value.code == L.ERR_INVALID_VALUE
+
+
+def test_gemm_on_a_created_stream(gpu, orc):
+    """A tiled GEMM and a split-K GEMM launched on a Stream object (not the default stream)."""
+    g = orc.GemmDesc(M=256, N=256, K=512)
+    A, B, C = _inputs(orc, g, 680)
+    ref = orc.gemm_f64(g, A, B, C)
+    s = gpu.Stream()
+    dA, dB, dC = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(C)
+    for launch in (lambda d: gpu.GEMM.gemm(dA, dB, dC, d, gpu.GEMM.make_desc(256, 256, 512), stream=s),
+                   lambda d: gpu.GEMM.gemm_splitk(dA, dB, dC, d, gpu.GEMM.make_desc(256, 256, 512), 2, stream=s)):
+        dD = gpu.DeviceArray(np.zeros(256 * 256, dtype=F32))
+        ws = launch(dD)
+        s.synchronize()
+        assert orc.normalized_error(g, dD.to_host(), ref) <= TIGHT_F32
+        del ws
