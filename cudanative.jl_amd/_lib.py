@@ -134,6 +134,8 @@ SIGNATURES = {
     "miw_gemm_acc_chunk": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
     "miw_gemm_splitk_workspace": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
     "miw_gemm_splitk": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
+    "miw_gemm_splitk_static": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _i, _vp]),
+    "miw_gemm_splitk_static_capacity": (_sz, []),
     "miw_gemm_bench": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _vp, _i, _i, ctypes.POINTER(_f)]),
     "miw_launch_overhead_probe": (_i, [_i, _i, ctypes.POINTER(_f), ctypes.POINTER(_f)]),
     "miw_mfma_power_probe": (_i, [_i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), _vp]),

@@ -168,6 +168,7 @@ bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f
 }
 
 int g_cu_count = 0;
+int splitk_scratch(void **out);  // address of the current device's static split-K workspace (below)
 
 int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
 {
@@ -249,6 +250,8 @@ int miw_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(MIW_ERR_UNSUPPORTED, "init: kernels are built for gfx950, device is %s", prop.gcnArchName);
     g_cu_count = prop.multiProcessorCount;
+    void *scratch = nullptr;
+    if (int rc = splitk_scratch(&scratch)) return rc;  // once per device, with that device current
     g_initialized.store(true, std::memory_order_release);
     g_err[0] = 0;
     return 0;
@@ -583,6 +586,32 @@ int miw_gemm(const miw_gemm_desc *desc, const void *A, const void *B, const void
 
 namespace {
 
+// Static workspace of miw_gemm_splitk_static: the Float32 partial products of one split-K GEMM.
+// Every GPU the library runs on holds its own copy from the time the library's code is loaded
+// there until the process ends.  In host code the array's name is not a device address: host code
+// uses the address hipGetSymbolAddress returned for the current device.
+constexpr size_t SPLITK_STATIC_BYTES = 32u << 20;
+static __device__ __align__(256) unsigned char g_splitk_scratch[SPLITK_STATIC_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void *> g_splitk_scratch_ptr[MAX_DEVICES];
+
+// Address of the current device's copy of the static workspace (looked up once per device).
+int splitk_scratch(void **out)
+{
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(MIW_ERR_UNSUPPORTED, "gemm_splitk_static: device index %d out of range", dev);
+    void *ptr = g_splitk_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_splitk_scratch)));
+        if (!ptr) return fail(MIW_ERR_UNSUPPORTED, "gemm_splitk_static: no address for the static workspace");
+        g_splitk_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return 0;
+}
+
 struct splitk_plan {
     miw::gemm_params full;   // the caller's problem
     miw::gemm_params slice;  // first pass: `splits` independent products of K / splits k-values each
@@ -702,6 +731,24 @@ int miw_gemm_splitk(const miw_gemm_desc *desc, const void *A, const void *B, con
     REQUIRE_INIT("gemm_splitk");
     return run_splitk(desc, plan, workspace, as_stream(stream));
 }
+
+int miw_gemm_splitk_static(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
+                           void *stream)
+{
+    splitk_plan plan;
+    if (int rc = plan_splitk(desc, A, B, C, D, splits, &plan)) return rc;
+    if (plan.bytes > SPLITK_STATIC_BYTES)
+        return fail(MIW_ERR_UNSUPPORTED,
+                    "gemm_splitk_static: %d slices of %lld x %lld Float32 need %zu bytes, the static workspace holds %zu; "
+                    "use miw_gemm_splitk with a workspace of your own",
+                    plan.splits, (long long)plan.full.M, (long long)plan.full.N, plan.bytes, SPLITK_STATIC_BYTES);
+    REQUIRE_INIT("gemm_splitk_static");
+    void *ws = nullptr;
+    if (int rc = splitk_scratch(&ws)) return rc;
+    return run_splitk(desc, plan, ws, as_stream(stream));
+}
+
+size_t miw_gemm_splitk_static_capacity(void) { return SPLITK_STATIC_BYTES; }
 
 int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream,
                    int warmup, int iters, float *ms_each)

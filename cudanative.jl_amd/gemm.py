@@ -68,6 +68,17 @@ def gemm_splitk(A, B, C, D, desc, splits=0, workspace=None, stream=None):
     return workspace
 
 
+def gemm_splitk_static(A, B, C, D, desc, splits=0, stream=None):
+    """gemm_splitk through the library's static device workspace: allocates nothing (at most
+    splitk_static_capacity() bytes of slices; calls that overlap on one GPU race)."""
+    _lib.check(_lib.load().miw_gemm_splitk_static(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), splits,
+                                                  _stream(stream)))
+
+
+def splitk_static_capacity():
+    return _lib.load().miw_gemm_splitk_static_capacity()
+
+
 def gemm_bench(A, B, C, D, desc, warmup=5, iters=20, stream=None):
     """Per-launch durations in milliseconds, HIP events on the launch stream."""
     ms = (ctypes.c_float * iters)()

@@ -220,6 +220,19 @@ int miw_gemm_splitk_workspace(const miw_gemm_desc *desc, int splits, int *splits
 int miw_gemm_splitk(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* miw_gemm_splitk for callers that cannot allocate device memory (code under HIP graph capture,
+   tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+   Same kernels and results as miw_gemm_splitk, with the slices going through a workspace that is
+   part of the library's device code: miw_gemm_splitk_static_capacity() bytes (32 MiB) that every
+   GPU the library runs on holds until the process ends.  It calls no hipMalloc, hipFree or other
+   allocating routine, and refuses (MIW_ERR_UNSUPPORTED) a problem whose splits * m * n * 4 bytes
+   exceed the capacity.  All calls on one GPU share that GPU's workspace: calls that overlap on one
+   GPU (two streams, two host threads) race; calls on one stream are ordered and safe.  Nothing in
+   the workspace needs clearing: the first pass writes every element the second pass reads. */
+int miw_gemm_splitk_static(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
+                           void *stream);
+size_t miw_gemm_splitk_static_capacity(void);
+
 /* warmup untimed launches, then iters launches each bracketed by HIP events on
    `stream`; ms_each[i] receives launch i's duration in milliseconds. */
 int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D,
