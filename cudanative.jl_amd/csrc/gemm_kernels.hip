@@ -3,6 +3,7 @@
 // gemm_tile_*.hip translation units (one per tile family, so that they build in parallel).
 #include "gemm_tiled.hpp"
 
+#include <cstdlib>
 #include <mutex>
 #include <unordered_map>
 
@@ -21,6 +22,9 @@ static const tiled_variant g_variants[] = {
     {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2, 0},
     {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, 4, 4 * (64 + 64) * KGRAN * 2, 0},
     {"tile256x256_pingpong", 256, 256, KGRAN, 2, 4, 3, 160 * 1024, 1},
+    {"tile256x128_pingpong", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 2},
+    {"tile128x256_pingpong", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 2},
+    {"tile128x128_pingpong", 128, 128, KGRAN, 4, 2, 4, 4 * (128 + 128) * KGRAN * 2, 2},
 };
 
 int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }
@@ -29,7 +33,8 @@ int tiled_f16acc_chunk() { return KGRAN; }
 bool tiled_supports_f16acc(int i)
 {
     const tiled_variant &v = g_variants[i];
-    if (v.pingpong) return false;  // fp32 accumulation only
+    if (v.pingpong == 1) return false;  // 32-k clusters: fp32 accumulation only
+    if (v.pingpong == 2) return true;   // 64-k clusters round in the memory cluster
     return waves_per_simd(v.bm, v.bn, v.wm * v.wn * 64) >= 2;
 }
 
@@ -44,6 +49,7 @@ const void *tiled_kernel_128x128_w2x2(bool xk, bool yk, int c_type, int d_type, 
 const void *tiled_kernel_64x64_w2x2(bool xk, bool yk, int c_type, int d_type, bool f16acc);
 const void *pp_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type);
 int pp_lds(int bm, int bn, bool xk, bool yk);
+const void *pp64_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type, bool f16acc);
 
 // Tile shape in canonical (I, J) terms: bm applies to I, bn to J.
 static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, bool f16acc)
@@ -58,6 +64,7 @@ static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, 
         case 6: return tiled_kernel_128x128_w2x2(xk, yk, c_type, d_type, f16acc);
         case 7: return tiled_kernel_64x64_w2x2(xk, yk, c_type, d_type, f16acc);
         case 8: return f16acc ? nullptr : pp_kernel(256, 256, xk, yk, c_type, d_type);
+        case 9: case 10: case 11: return pp64_kernel(g_variants[i].bm, g_variants[i].bn, xk, yk, c_type, d_type, f16acc);
     }
     return nullptr;
 }
@@ -82,7 +89,7 @@ static void canonical_layout(const gemm_params &g, bool *xk, bool *yk)
 
 bool tiled_supports_layout(int i, const gemm_params &g)
 {
-    if (!g_variants[i].pingpong) return true;
+    if (g_variants[i].pingpong != 1) return true;
     bool xk, yk;
     canonical_layout(g, &xk, &yk);
     return pp_kernel(g_variants[i].bm, g_variants[i].bn, xk, yk, 1, 1) != nullptr;  // two K-major 256-row rings do not fit in LDS
@@ -135,9 +142,16 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
     while ((gi * 2) * (gi * 2) <= per_xcd) gi *= 2;
     p.group_i = gi < p.tiles_i ? gi : p.tiles_i;
 
+#ifdef MIW_PP_TS
+    // measurement builds: device address of the timestamp buffer, in hexadecimal
+    p.ts = nullptr;
+    if (const char *e = getenv("MIW_TS")) p.ts = (long long *)strtoull(e, nullptr, 16);
+#endif
     const void *fn = pick_kernel(i, xk, yk, c_type, d_type, f16acc);
     if (!fn) return hipErrorInvalidValue;
-    const int lds_bytes = v.pingpong ? pp_lds(v.bm, v.bn, xk, yk) : v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
+    const int lds_bytes = v.pingpong == 1 ? pp_lds(v.bm, v.bn, xk, yk)
+                          : v.pingpong == 2 ? v.lds_bytes
+                                            : v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
     hipError_t e = allow_dynamic_lds(fn, lds_bytes);
     if (e != hipSuccess) return e;
     void *args[] = {&p};

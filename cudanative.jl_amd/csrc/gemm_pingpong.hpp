@@ -36,6 +36,18 @@ namespace miw {
 #define MIW_PP_ABLATE 0
 #endif
 
+// Second measurement switch (off in every shipped build; gemm_kernels.hip must be compiled with it
+// too): with MIW_PP_TS the 64-k-cluster kernel records, per wavefront, the shader clock at kernel
+// entry [0], after the prologue's loads have landed [1], at the middle of the loop [2], one pair
+// later [3], at the end of the loop [4], when the last store is issued [5] and when the stores have
+// drained [6], plus the 100 MHz wall clock at exit [7] and entry [8], into the buffer whose device
+// address the environment variable MIW_TS holds.
+#ifdef MIW_PP_TS
+#define MIW_PP_STAMP(i) { __builtin_amdgcn_sched_barrier(0); ts[i] = clock64(); __builtin_amdgcn_sched_barrier(0); }
+#else
+#define MIW_PP_STAMP(i)
+#endif
+
 constexpr int PP_KMAJOR_SLOTS = 3;
 constexpr int PP_IMAJOR_ENTRIES = 4;
 
@@ -447,6 +459,393 @@ void k_gemm_pp(tiled_params p)
     if (!p.use_c || fold_c) epilogue(false, false);
     else if (p.c_trans) epilogue(true, true);
     else epilogue(true, false);
+}
+
+// ---------------------------------------------------------------------------
+// Ping-pong kernel with clusters of 64 k-values (one LDS slot), for the tiles whose rings of whole
+// slots fit in LDS: 256x128, 128x256 (three slots) and 128x128 (four).  A wavefront's memory
+// cluster reads the fragments of both k-steps of pair p out of the pair's slot and requests pair
+// p + NSLOT - 1 into the slot of pair p - 1 (which the other group finished reading one barrier
+// ago); its compute cluster issues the pair's 2 * TI * TJ MFMAs.  At the end of the memory cluster
+// the wavefront lets the NSLOT - 2 youngest pairs stay in flight: pair p + 1 has landed, and the
+// two barriers that follow publish it before anyone reads it.  Both operand kinds use the slot
+// layouts, loaders and fragment readers of gemm_tiled.hpp.
+//
+// fp16 accumulation rounds the running sums to Float16 once per slot (64 k-values): a tile is
+// rounded two MFMAs after its last MFMA of the pair, inside the compute cluster (the memory
+// cluster is the longer of the two: the LDS serves 128 bytes a clock and is the unit these tiles
+// keep busiest).  The C operand is requested before anything else, converted once the prologue's
+// loads have landed and added at the first rounding: acc = half(half(beta * C) + sum of the first
+// 64 k-values), so that its latency hides behind the prologue.
+template <int BI, int BJ, int WI, int WJ, int NSLOT, bool XK, bool YK, class CT, class DT, bool F16ACC>
+__global__ __launch_bounds__(WI *WJ * 64) __attribute__((amdgpu_waves_per_eu(2)))
+void k_gemm_pp64(tiled_params p)
+{
+    constexpr int NT = WI * WJ * 64;
+    static_assert(NT == 512, "two wavefronts per SIMD");
+    constexpr int WTI = BI / WI, WTJ = BJ / WJ;
+    constexpr int TI = WTI / 16, TJ = WTJ / 16;
+    constexpr int XBYTES = BI * KGRAN * 2, YBYTES = BJ * KGRAN * 2, SLOT = XBYTES + YBYTES;
+    static_assert(NSLOT >= 3 && NSLOT * SLOT <= 160 * 1024, "ring does not fit in LDS");
+    using xload = slot_loader<BI, XK, NT>;
+    using yload = slot_loader<BJ, YK, NT>;
+    constexpr int NLX = xload::NLOAD, NLY = yload::NLOAD, LPAIR = NLX + NLY;  // loads per thread and pair
+    constexpr int NTILE = TI * TJ;
+    constexpr int NFRAG = 2 * (TI + TJ);  // fragment units of a memory cluster
+
+#ifdef MIW_PP_TS
+    long long ts[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    ts[0] = clock64();
+    ts[8] = wall_clock64();
+#endif
+    extern __shared__ __attribute__((aligned(128))) char smem[];
+    MIW_LDS char *lds = (MIW_LDS char *)smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wi = wave % WI, wj = wave / WI;
+    const bool late_group = wave >= 4;
+
+    // Workgroup -> tile, as in k_gemm_tiled.
+    int tile_id;
+    {
+        const int total = p.tiles_i * p.tiles_j;
+        const int pid = blockIdx.x;
+        const int per = total >> 3, rem = total & 7;
+        const int xcd = pid & 7, loc = pid >> 3;
+        tile_id = xcd < rem ? xcd * (per + 1) + loc : rem * (per + 1) + (xcd - rem) * per + loc;
+    }
+    int ti0, tj0;
+    {
+        const int gsz = p.group_i * p.tiles_j;
+        const int gid = tile_id / gsz;
+        const int first = gid * p.group_i;
+        const int gi = min(p.tiles_i - first, p.group_i);
+        const int in = tile_id - gid * gsz;
+        ti0 = first + in % gi;
+        tj0 = in / gi;
+    }
+    const long bt = blockIdx.y;
+    const int i0 = ti0 * BI, j0 = tj0 * BJ;
+
+    const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
+    const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);
+    const long xstep = XK ? KGRAN : (long)KGRAN * p.ldx;
+    const long ystep = YK ? KGRAN : (long)KGRAN * p.ldy;
+    const unsigned xoff = xload::lane_offset(tid, (int)p.ldx);
+    const unsigned yoff = yload::lane_offset(tid, (int)p.ldy);
+
+    frag_reader<BI, XK> xr;
+    frag_reader<BJ, YK> yr;
+    xr.init(wi * WTI, lane);
+    yr.init(wj * WTJ, lane);
+
+    const int q = lane >> 4, r = lane & 15;
+    const int row = i0 + wi * WTI + 4 * q;  // + 16*ti
+    const int col = j0 + wj * WTJ + r;      // + 16*tj
+    const CT *C = (const CT *)p.C + bt * p.sc;
+    DT *D = (DT *)p.D + bt * p.sd;
+
+    float4_t acc[TI][TJ];
+#pragma unroll
+    for (int a = 0; a < TI; a++)
+#pragma unroll
+        for (int b = 0; b < TJ; b++) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto read_c = [&](int a, int b, bool trans) -> float4_t {
+        float4_t c;
+        const int ii = row + 16 * a, jj = col + 16 * b;
+        if (trans) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) c[v] = (float)C[(long)(ii + v) * p.ldc + jj];
+        } else if constexpr (__is_same(CT, float)) {
+            c = *(const float4_t *)(C + (long)jj * p.ldc + ii);
+        } else {
+            half4_t h = *(const half4_t *)(C + (long)jj * p.ldc + ii);
+            c = float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+        }
+        return c;
+    };
+
+    const int NP = p.K / KGRAN;
+    const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
+    int next = 0;          // next pair to request
+    int wslot = 0;         // the slot it goes to
+    unsigned dma_dst = 0;  // this wavefront's first destination byte in that slot
+    auto begin_request = [&]() { dma_dst = wave_dst + (unsigned)(wslot * SLOT); };
+    auto request_one = [&]<int I>(std::integral_constant<int, I>) {
+        if constexpr (I < NLX)
+            lds_dma16(X + xload::load_delta(I, p.ldx), xoff, dma_dst + (unsigned)(I * NT * 16));
+        else
+            lds_dma16(Y + yload::load_delta(I - NLX, p.ldy), yoff, dma_dst + XBYTES + (unsigned)((I - NLX) * NT * 16));
+    };
+    // Past the end of K the last pair is requested again, into a slot nobody reads any more.
+    auto end_request = [&]() {
+        next++;
+        wslot = wslot + 1 == NSLOT ? 0 : wslot + 1;
+        const bool more = next < NP;
+        X += more ? xstep : 0;
+        Y += more ? ystep : 0;
+    };
+
+    // fp16 accumulation: the C operand is requested first, as raw bits that no instruction touches
+    // before the prologue's wait (a conversion here would make the compiler wait for the loads
+    // before the first direct-to-LDS load is issued).  C laid out as D: the lane's four halves in two
+    // registers; C stored across D: one zero-extended half per register.
+    unsigned craw[F16ACC ? TI : 1][F16ACC ? TJ : 1][4];
+    if constexpr (F16ACC) {
+        if (p.use_c) {
+            auto fetch = [&]<bool TRANS>(std::bool_constant<TRANS>) {
+#pragma unroll
+                for (int a = 0; a < TI; a++)
+#pragma unroll
+                    for (int b = 0; b < TJ; b++) {
+                        const int ii = row + 16 * a, jj = col + 16 * b;
+                        if constexpr (TRANS) {
+#pragma unroll
+                            for (int v = 0; v < 4; v++) craw[a][b][v] = *(const unsigned short *)(C + (long)(ii + v) * p.ldc + jj);
+                        } else {
+                            const uint2_t two = *(const uint2_t *)(C + (long)jj * p.ldc + ii);
+                            craw[a][b][0] = two[0];
+                            craw[a][b][1] = two[1];
+                        }
+                    }
+            };
+            if (p.c_trans) fetch(std::true_type{});
+            else fetch(std::false_type{});
+        }
+    }
+    // Prologue: the first NSLOT - 1 pairs.
+#pragma unroll
+    for (int s = 0; s < NSLOT - 1; s++) {
+        begin_request();
+        [&]<int... I>(std::integer_sequence<int, I...>) { (request_one(std::integral_constant<int, I>{}), ...); }
+        (std::make_integer_sequence<int, LPAIR>{});
+        end_request();
+    }
+    wait_loads_and_barrier<0>();
+    float4_t cinit[F16ACC ? TI : 1][F16ACC ? TJ : 1];
+    if constexpr (F16ACC) {
+        auto convert = [&]<bool TRANS>(std::bool_constant<TRANS>) {
+#pragma unroll
+            for (int a = 0; a < TI; a++)
+#pragma unroll
+                for (int b = 0; b < TJ; b++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const unsigned bits = TRANS ? craw[a][b][v] : craw[a][b][v >> 1] >> (16 * (v & 1));
+                        const float c = (float)__builtin_bit_cast(half_t, (unsigned short)bits);
+                        cinit[a][b][v] = round_through_half(p.beta * c);
+                    }
+        };
+        if (!p.use_c) {
+#pragma unroll
+            for (int a = 0; a < TI; a++)
+#pragma unroll
+                for (int b = 0; b < TJ; b++) cinit[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+        } else if (p.c_trans) {
+            convert(std::true_type{});
+        } else {
+            convert(std::false_type{});
+        }
+    }
+
+    half8_t fx[2][TI], fy[2][TJ];
+    if constexpr (MIW_PP_ABLATE & 2) {
+        [&]<int... U>(std::integer_sequence<int, U...>) { ((fx[0][U] = fx[1][U] = xr.template read<U, 0>(lds)), ...); }(std::make_integer_sequence<int, TI>{});
+        [&]<int... U>(std::integer_sequence<int, U...>) { ((fy[0][U] = fy[1][U] = yr.template read<U, 0>(lds + XBYTES)), ...); }(std::make_integer_sequence<int, TJ>{});
+    }
+    // Rounding of the tile MFMA number m of a k-step works on.  FIRST: the pair's sums meet the C operand here.
+    auto round_tile = [&]<bool FIRST>(int m, std::bool_constant<FIRST>) {
+        const int a = m / TJ, b = serpentine_column(m, TJ);
+        float4_t v = acc[a][b];
+        if constexpr (FIRST) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] += cinit[a][b][e];
+        }
+        half4_t h = __builtin_convertvector(v, half4_t);
+        acc[a][b] = __builtin_convertvector(h, float4_t);
+    };
+    // Fragment unit U of a memory cluster (step 0: the TI x-fragments, then the TJ y-fragments; then
+    // step 1), preceded by the direct-to-LDS loads that go out before it (load n before unit
+    // n * NFRAG / LPAIR).
+    auto cluster_unit = [&]<int U>(MIW_LDS const char *xs, std::integral_constant<int, U>) {
+        [&]<int... N>(std::integer_sequence<int, N...>) {
+            (([&] {
+                 if constexpr (N * NFRAG / LPAIR == U && !(MIW_PP_ABLATE & 1)) {
+                     request_one(std::integral_constant<int, N>{});
+                     __builtin_amdgcn_sched_barrier(0);
+                 }
+             }()),
+             ...);
+        }(std::make_integer_sequence<int, LPAIR>{});
+        constexpr int H = U / (TI + TJ), V = U % (TI + TJ);
+        if constexpr (MIW_PP_ABLATE & 2) {
+            asm volatile("" : "+v"(fx[H][V % TI]), "+v"(fy[H][V % TJ]));
+        } else {
+            if constexpr (V < TI) fx[H][V] = xr.template read<V, H>(xs);
+            else fy[H][V - TI] = yr.template read<V - TI, H>(xs + XBYTES);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int rslot = 0;
+    auto memory_cluster = [&]() {
+        MIW_LDS const char *xs = lds + rslot * SLOT;
+        begin_request();
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            (cluster_unit(xs, std::integral_constant<int, U>{}), ...);
+        }(std::make_integer_sequence<int, NFRAG>{});
+        end_request();
+        rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // RMODE 0: fp32 sums; 1: round every tile to Float16 ROUND_LAG MFMAs after its last MFMA of the
+    // pair; 2: the same for the first pair, which adds the C operand.
+    constexpr int ROUND_LAG = 2;
+    auto compute_cluster = [&]<int RMODE>(std::integral_constant<int, RMODE>) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int m = 0; m < NTILE; m++) {
+                // serpentine order: every MFMA changes exactly one of its two operand fragments
+                const int a = m / TJ, b = serpentine_column(m, TJ);
+                if constexpr (!(MIW_PP_ABLATE & 4)) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], acc[a][b], 0, 0, 0);
+                if constexpr (RMODE != 0)
+                    if (h == 1 && m >= ROUND_LAG) round_tile(m - ROUND_LAG, std::bool_constant<RMODE == 2>{});
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        if constexpr (RMODE != 0)
+#pragma unroll
+            for (int m = NTILE > ROUND_LAG ? NTILE - ROUND_LAG : 0; m < NTILE; m++) round_tile(m, std::bool_constant<RMODE == 2>{});
+    };
+
+    // Folding C (Float32 C laid out as D, alpha == 1): CPT MFMA tiles per cluster over the last
+    // NFOLD clusters, requested at the end of a memory cluster with ordinary loads into registers
+    // (the lane fetches the 16 bytes it owns).  They are the youngest loads of their cluster; the
+    // wait LAG clusters later covers them and that cluster adds them in, so C has LAG clusters of
+    // both wavefront groups to arrive.  LAG + 1 register stages rotate.
+    constexpr int CPT = 1;
+    constexpr int NFOLD = NTILE / CPT;
+    constexpr int LAG = NSLOT - 1;
+    constexpr bool CAN_FOLD = !F16ACC && __is_same(CT, float) && TI % CPT == 0;
+    bool fold_c = false;
+    if constexpr (CAN_FOLD) fold_c = p.use_c && !p.c_trans && p.alpha == 1.0f && NP >= NFOLD + 1 && p.ldc < (1l << 22);
+    float4_t cst[LAG + 1][CPT];
+    const char *cnext = (const char *)(C + (long)j0 * p.ldc + i0);
+    const unsigned coff = 4u * (unsigned)((wj * WTJ + r) * (int)p.ldc + wi * WTI + 4 * q);
+    auto fold_request = [&]<int S>(std::integral_constant<int, S>) {
+        [&]<int... U>(std::integer_sequence<int, U...>) {
+            (([&] {
+                 constexpr int a = (S * CPT + U) % TI;
+                 asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(cst[S % (LAG + 1)][U]) : "v"(coff), "s"(cnext), "n"(64 * a) : "memory");
+                 if constexpr (a == TI - 1) cnext += 64 * p.ldc;
+             }()),
+             ...);
+        }(std::make_integer_sequence<int, CPT>{});
+    };
+    auto fold_add = [&]<int S>(std::integral_constant<int, S>) {
+#pragma unroll
+        for (int u = 0; u < CPT; u++) {
+            const int a = (S * CPT + u) % TI, b = (S * CPT + u) / TI;
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[a][b][e] = __builtin_fmaf(p.beta, cst[S % (LAG + 1)][u][e], acc[a][b][e]);
+        }
+    };
+    // One pair: memory cluster, barrier, compute cluster, barrier.  FS >= 0: fold cluster FS.
+    auto pair = [&]<int FS, int RMODE>(std::integral_constant<int, FS>, std::integral_constant<int, RMODE> rmode) {
+        memory_cluster();
+        if constexpr (FS >= 0) {
+            fold_request(std::integral_constant<int, FS>{});
+            __builtin_amdgcn_sched_barrier(0);
+            // Allowed to stay in flight: the ring loads of the NSLOT - 2 youngest clusters with the fold
+            // loads issued after them, and the fold loads of the cluster before those (younger than
+            // that cluster's ring loads, which must have landed).
+            constexpr int YOUNGER = (NSLOT - 2) * LPAIR + CPT * (FS + 1 < NSLOT - 1 ? FS + 1 : NSLOT - 1);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt((YOUNGER & 15) | (7 << 4) | (0 << 8) | ((YOUNGER >> 4) << 14));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (FS >= LAG) fold_add(std::integral_constant<int, FS - LAG>{});
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
+        }
+        compute_cluster(rmode);
+        __builtin_amdgcn_s_barrier();
+    };
+    constexpr std::integral_constant<int, -1> no_fold{};
+    constexpr std::integral_constant<int, 0> plain{};
+
+    MIW_PP_STAMP(1)
+    if (late_group) __builtin_amdgcn_s_barrier();
+    const int NPM = fold_c ? NP - NFOLD : NP;
+    if (NPM > 0) pair(no_fold, std::integral_constant<int, F16ACC ? 2 : 0>{});
+    for (int pr = 1; pr < NPM; pr++) {
+#ifdef MIW_PP_TS
+        if (pr == NPM / 2) MIW_PP_STAMP(2)
+        if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
+#endif
+        pair(no_fold, std::integral_constant<int, F16ACC ? 1 : 0>{});
+    }
+    MIW_PP_STAMP(9)
+    if constexpr (CAN_FOLD) {
+        if (fold_c) {
+            [&]<int... G>(std::integer_sequence<int, G...>) {
+                (pair(std::integral_constant<int, G>{}, plain), ...);
+            }(std::make_integer_sequence<int, NFOLD>{});
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may outlive the workgroup's LDS
+    if constexpr (CAN_FOLD) {
+        if (fold_c) {
+            [&]<int... G>(std::integer_sequence<int, G...>) {
+                (fold_add(std::integral_constant<int, NFOLD - LAG + G>{}), ...);
+            }(std::make_integer_sequence<int, LAG>{});
+        }
+    }
+    if (!late_group) __builtin_amdgcn_s_barrier();
+    MIW_PP_STAMP(4)
+
+    // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
+    auto epilogue = [&](bool with_c, bool trans) {
+#pragma unroll
+        for (int b = 0; b < TJ; b++)
+#pragma unroll
+            for (int a = 0; a < TI; a++) {
+                float4_t v = acc[a][b];
+                if constexpr (!F16ACC) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] *= p.alpha;
+                    if (with_c) {
+                        float4_t c = read_c(a, b, trans);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
+                    }
+                }
+                DT *dst = D + (long)(col + 16 * b) * p.ldd + (row + 16 * a);
+                if constexpr (__is_same(DT, float)) {
+                    *(float4_t *)dst = v;
+                } else {
+                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    *(half4_t *)dst = h;
+                }
+            }
+    };
+    if (F16ACC || !p.use_c || fold_c) epilogue(false, false);
+    else if (p.c_trans) epilogue(true, true);
+    else epilogue(true, false);
+#ifdef MIW_PP_TS
+    MIW_PP_STAMP(5)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    MIW_PP_STAMP(6)
+    ts[7] = wall_clock64();
+    if (p.ts && lane == 0)
+        for (int i = 0; i < 10; i++) p.ts[((long)(blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 10 + i] = ts[i];
+#endif
 }
 
 }  // namespace miw

@@ -70,6 +70,9 @@ struct tiled_params {
     int use_c;
     float alpha, beta;
     int tiles_i, tiles_j, group_i;
+#ifdef MIW_PP_TS
+    long long *ts;  // measurement builds: 10 counters per wavefront (see k_gemm_pp64), or null
+#endif
 };
 
 // s_waitcnt vmcnt(N) lgkmcnt(0); s_barrier.  The direct-to-LDS loads are issued

@@ -43,7 +43,8 @@ const char *frag_kernel_name(int i);
 struct tiled_variant {
     const char *name;
     int bm, bn, bk, wm, wn, stages, lds_bytes;
-    int pingpong;  // 1: the two wavefronts of a SIMD alternate between MFMA and memory clusters (gemm_pingpong.hpp)
+    int pingpong;  // the two wavefronts of a SIMD alternate between MFMA and memory clusters (gemm_pingpong.hpp):
+                   // 1: clusters of 32 k-values, 2: of 64; 0: the pipelined kernel of gemm_tiled.hpp
 };
 int tiled_variant_count();
 const tiled_variant &tiled_variant_at(int i);
