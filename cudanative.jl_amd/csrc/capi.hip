@@ -183,7 +183,7 @@ int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc,
     std::stable_sort(order.begin(), order.end(), [](int a, int b) {
         const miw::tiled_variant &va = miw::tiled_variant_at(a), &vb = miw::tiled_variant_at(b);
         if (va.bm * va.bn != vb.bm * vb.bn) return va.bm * va.bn > vb.bm * vb.bn;
-        return va.pingpong > vb.pingpong;
+        return va.kind > vb.kind;
     });
     for (int i : order) {
         if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk)) continue;
@@ -529,7 +529,7 @@ int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out)
     out->block_m = v.bm; out->block_n = v.bn; out->block_k = v.bk;
     out->waves_m = v.wm; out->waves_n = v.wn; out->stages = v.stages; out->lds_bytes = v.lds_bytes;
     out->f16_accumulate = miw::tiled_supports_f16acc(variant - 1) ? 1 : 0;
-    out->pingpong = v.pingpong;
+    out->pingpong = v.kind == miw::KIND_PINGPONG32 || v.kind == miw::KIND_PINGPONG64;
     return 0;
 }
 

@@ -12,7 +12,7 @@ namespace miw {
 // --------------------------------------------------------------- variants --
 
 static const tiled_variant g_variants[] = {
-    // name                    bm   bn  bk     wm wn slots lds (pingpong: ring depth of a K-major operand, largest ring)
+    // name                    bm   bn  bk     wm wn slots lds, kind (32-k ping-pong: ring depth of a K-major operand, largest ring)
     {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2, 0},
     {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2, 0},
     {"tile256x128_w4x2", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 0},
@@ -33,8 +33,8 @@ int tiled_f16acc_chunk() { return KGRAN; }
 bool tiled_supports_f16acc(int i)
 {
     const tiled_variant &v = g_variants[i];
-    if (v.pingpong == 1) return false;  // 32-k clusters: fp32 accumulation only
-    if (v.pingpong == 2) return true;   // 64-k clusters round in the memory cluster
+    if (v.kind == KIND_PINGPONG32) return false;  // 32-k clusters: fp32 accumulation only
+    if (v.kind == KIND_PINGPONG64) return true;   // 64-k clusters round in the compute cluster
     return waves_per_simd(v.bm, v.bn, v.wm * v.wn * 64) >= 2;
 }
 
@@ -50,6 +50,7 @@ const void *tiled_kernel_64x64_w2x2(bool xk, bool yk, int c_type, int d_type, bo
 const void *pp_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type);
 int pp_lds(int bm, int bn, bool xk, bool yk);
 const void *pp64_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type, bool f16acc);
+
 
 // Tile shape in canonical (I, J) terms: bm applies to I, bn to J.
 static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, bool f16acc)
@@ -89,7 +90,7 @@ static void canonical_layout(const gemm_params &g, bool *xk, bool *yk)
 
 bool tiled_supports_layout(int i, const gemm_params &g)
 {
-    if (g_variants[i].pingpong != 1) return true;
+    if (g_variants[i].kind != KIND_PINGPONG32) return true;
     bool xk, yk;
     canonical_layout(g, &xk, &yk);
     return pp_kernel(g_variants[i].bm, g_variants[i].bn, xk, yk, 1, 1) != nullptr;  // two K-major 256-row rings do not fit in LDS
@@ -149,9 +150,9 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
 #endif
     const void *fn = pick_kernel(i, xk, yk, c_type, d_type, f16acc);
     if (!fn) return hipErrorInvalidValue;
-    const int lds_bytes = v.pingpong == 1 ? pp_lds(v.bm, v.bn, xk, yk)
-                          : v.pingpong == 2 ? v.lds_bytes
-                                            : v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
+    const int lds_bytes = v.kind == KIND_PINGPONG32 ? pp_lds(v.bm, v.bn, xk, yk)
+                          : v.kind != KIND_PIPELINED ? v.lds_bytes
+                                                     : v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
     hipError_t e = allow_dynamic_lds(fn, lds_bytes);
     if (e != hipSuccess) return e;
     void *args[] = {&p};

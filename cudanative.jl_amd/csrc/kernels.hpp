@@ -40,11 +40,16 @@ int frag_kernel_count();
 const char *frag_kernel_name(int i);
 
 // --- gemm_kernels.hip
+// Kernel families of the LDS-tiled GEMM.
+enum {
+    KIND_PIPELINED = 0,   // gemm_tiled.hpp: every wavefront overlaps its own loads, LDS reads and MFMAs
+    KIND_PINGPONG32 = 1,  // gemm_pingpong.hpp: the two wavefronts of a SIMD alternate between MFMA and memory clusters of 32 k-values
+    KIND_PINGPONG64 = 2   // the same with clusters of 64 k-values
+};
 struct tiled_variant {
     const char *name;
     int bm, bn, bk, wm, wn, stages, lds_bytes;
-    int pingpong;  // the two wavefronts of a SIMD alternate between MFMA and memory clusters (gemm_pingpong.hpp):
-                   // 1: clusters of 32 k-values, 2: of 64; 0: the pipelined kernel of gemm_tiled.hpp
+    int kind;  // KIND_*
 };
 int tiled_variant_count();
 const tiled_variant &tiled_variant_at(int i);

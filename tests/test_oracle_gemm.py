@@ -108,6 +108,43 @@ def test_f16acc_intermediate_rounding_is_visible(orc):
     assert d[0, 0] == 0.5 * 2050 + 6
 
 
+@pytest.mark.parametrize("kc,K", [(16, 208), (64, 320), (64, 64 * 5 + 16)])
+def test_f16acc_multi_chunk_model_against_an_independent_float64_loop(orc, kc, K):
+    """Random fixed-point data (multiples of 2^-10 in [-1, 1]: every product and chunk sum is exact in
+    float64 whatever the order of summation), alpha and beta different from 1, several chunks with a
+    ragged last one, mixed layouts: miwo_gemm_f16acc must equal, bit for bit, a numpy loop written from
+    the definition  acc = half(beta*C); acc = half(acc + alpha * sum_chunk)  with one rounding per
+    chunk.  The variant that rounds alpha * sum to half on its own before the addition (a plausible
+    double rounding) is shown to give different bits on the same data, so the comparison can tell."""
+    rng = np.random.default_rng(1000 + kc + K)
+    M, N = 48, 32
+    alpha, beta = 0.75, -1.5
+    g = orc.GemmDesc(M=M, N=N, K=K, c_type=orc.F16, d_type=orc.F16, alpha=alpha, beta=beta, a_layout=orc.ROW,
+                     c_layout=orc.ROW, lda=K + 8, ldd=M + 16)
+    a = (rng.integers(-1024, 1025, (M, K)) / 1024.0).astype(np.float16)
+    b = (rng.integers(-1024, 1025, (K, N)) / 1024.0).astype(np.float16)
+    c = (rng.integers(-1024, 1025, (M, N)) / 1024.0).astype(np.float16)
+    A, B, C = orc.to_storage(a, orc.ROW, K + 8), orc.to_storage(b, orc.COL), orc.to_storage(c, orc.ROW)
+    got = orc.from_storage(orc.gemm_f16acc(g, kc, A, B, C), M, N, orc.COL, M + 16)
+
+    def half(x):
+        return x.astype(np.float16).astype(np.float64)
+
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    acc = half(beta * c.astype(np.float64))
+    wrong = acc.copy()
+    for k0 in range(0, K, kc):
+        s = a64[:, k0:k0 + kc] @ b64[k0:k0 + kc, :]
+        assert np.all(s * 2 ** 20 == np.round(s * 2 ** 20))          # exact: a multiple of 2^-20 below 2^8
+        acc = half(acc + alpha * s)
+        wrong = half(wrong + half(alpha * s))
+    assert np.array_equal(got.astype(np.float64), acc)
+    assert np.count_nonzero(wrong != acc) > 0
+    # and the rounding per chunk is visible: one rounding at the end gives other bits somewhere
+    once = half(half(beta * c.astype(np.float64)) + alpha * (a64 @ b64))
+    assert np.count_nonzero(once != acc) > 0
+
+
 def test_normalized_error_metric(orc):
     g = orc.GemmDesc(M=32, N=16, K=16, batch=2)
     A, B, C = _rand_problem(orc, g, 60)
