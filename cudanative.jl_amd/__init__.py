@@ -10,7 +10,7 @@ import ctypes as _ctypes
 from . import _lib
 from ._lib import MIWError, DeviceInfo
 from .array import AS, DeviceArray, DevicePtr, CU_NULL, pointer
-from .execution import HostKernel, Stream, cuda, cufunction, cudaconvert, kernel_names, synchronize
+from .execution import HostKernel, Module, Stream, cuda, cufunction, cudaconvert, kernel_names, synchronize
 from . import wmma as WMMA
 from . import gemm as GEMM
 from . import reflection

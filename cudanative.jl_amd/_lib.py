@@ -147,6 +147,9 @@ SIGNATURES = {
     "miw_kernel_attributes_get": (_i, [_vp, ctypes.POINTER(KernelAttributes)]),
     "miw_kernel_occupancy": (_i, [_vp, _sz, ctypes.POINTER(_i), ctypes.POINTER(_i)]),
     "miw_launch": (_i, [_vp, _u3, _u3, ctypes.c_uint, _vp, _vpp]),
+    "miw_module_load": (_i, [ctypes.c_char_p, _sz, _vpp]),
+    "miw_module_get_kernel": (_i, [_vp, ctypes.c_char_p, _vpp]),
+    "miw_module_unload": (_i, [_vp]),
 }
 
 _lib = None

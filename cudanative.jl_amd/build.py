@@ -13,8 +13,12 @@ LIB = os.path.join(HERE, "libmiwmma.so")
 SOURCES = ["gemm_tile_256x256_w2x4.hip", "gemm_tile_256x128.hip", "gemm_tile_256x256_w2x2.hip", "gemm_tile_small.hip", "gemm_tile_pp.hip", "gemm_tile_pp64.hip",
            "capi.hip", "frag_kernels.hip", "gemm_kernels.hip"]
 
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+EXAMPLE_SRC = os.path.join(HERE, "examples", "user_kernel.hip")
+EXAMPLE_CO = os.path.join(HERE, "examples", "user_kernel.hsaco")
+
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-I" + INCLUDE,
     "-Wall", "-Wextra", "-Wno-unused-command-line-argument", "-Wno-inline-asm",
     # keep the compiler from forming packed-fp32 VALU ops out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -50,7 +54,21 @@ def build(verbose=False, extra_flags=()):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    build_example(verbose)
     return LIB
+
+
+def build_example(verbose=False):
+    """The user-kernel example as a gfx950 code object, for miw_module_load."""
+    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++20", "--genco", "-I" + INCLUDE,
+           "-Wno-unused-command-line-argument", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           EXAMPLE_SRC, "-o", EXAMPLE_CO]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd), p.stdout))
+    return EXAMPLE_CO
 
 
 if __name__ == "__main__":

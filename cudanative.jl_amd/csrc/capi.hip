@@ -9,6 +9,8 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
+#include <unordered_map>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -168,6 +170,18 @@ bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f
 }
 
 int g_cu_count = 0;
+
+// Kernels of code objects the caller loaded (miw_module_load): handle -> module it belongs to.
+// miw_launch and the attribute queries tell them from the library's own kernels by this table.
+std::mutex g_module_mu;
+std::unordered_map<void *, void *> g_module_kernels;
+std::unordered_map<void *, int> g_modules;
+
+bool is_module_kernel(void *kernel)
+{
+    std::lock_guard<std::mutex> lock(g_module_mu);
+    return g_module_kernels.count(kernel) != 0;
+}
 int splitk_scratch(void **out);  // address of the current device's static split-K workspace (below)
 
 int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
@@ -929,6 +943,21 @@ int miw_kernel_attributes_get(void *kernel, miw_kernel_attributes *out)
 {
     if (!kernel || !out) return fail(MIW_ERR_NULL_POINTER, "kernel_attributes: null argument");
     REQUIRE_INIT("kernel_attributes");
+    if (is_module_kernel(kernel)) {
+        hipFunction_t f = (hipFunction_t)kernel;
+        int regs = 0, threads = 0, lds = 0, local = 0, cst = 0;
+        HIP_TRY(hipFuncGetAttribute(&regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, f));
+        HIP_TRY(hipFuncGetAttribute(&threads, HIP_FUNC_ATTRIBUTE_MAX_THREADS_PER_BLOCK, f));
+        HIP_TRY(hipFuncGetAttribute(&lds, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, f));
+        HIP_TRY(hipFuncGetAttribute(&local, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, f));
+        HIP_TRY(hipFuncGetAttribute(&cst, HIP_FUNC_ATTRIBUTE_CONST_SIZE_BYTES, f));
+        out->num_regs = regs;
+        out->max_threads_per_block = threads;
+        out->static_shared_bytes = (size_t)lds;
+        out->local_bytes = (size_t)local;
+        out->const_bytes = (size_t)cst;
+        return 0;
+    }
     hipFuncAttributes a;
     HIP_TRY(hipFuncGetAttributes(&a, kernel));
     out->num_regs = a.numRegs;
@@ -943,13 +972,87 @@ int miw_kernel_occupancy(void *kernel, size_t dynamic_shmem, int *min_grid, int 
 {
     if (!kernel || !min_grid || !block) return fail(MIW_ERR_NULL_POINTER, "kernel_occupancy: null argument");
     REQUIRE_INIT("kernel_occupancy");
+    if (is_module_kernel(kernel)) {
+        HIP_TRY(hipModuleOccupancyMaxPotentialBlockSize(min_grid, block, (hipFunction_t)kernel, dynamic_shmem, 0));
+        return 0;
+    }
     HIP_TRY(hipOccupancyMaxPotentialBlockSize(min_grid, block, kernel, dynamic_shmem, 0));
+    return 0;
+}
+
+int miw_module_load(const void *image, size_t bytes, void **module)
+{
+    if (!image || !module) return fail(MIW_ERR_NULL_POINTER, "module_load: null argument");
+    *module = nullptr;
+    // an ELF code object or a clang offload bundle that holds one
+    static const char bundle_magic[] = "__CLANG_OFFLOAD_BUNDLE__";
+    const bool elf = bytes >= 64 && memcmp(image, "\177ELF", 4) == 0;
+    const bool bundle = bytes >= sizeof(bundle_magic) - 1 && memcmp(image, bundle_magic, sizeof(bundle_magic) - 1) == 0;
+    if (!elf && !bundle)
+        return fail(MIW_ERR_INVALID_VALUE, "module_load: %zu bytes that are neither an ELF code object nor an offload bundle", bytes);
+    REQUIRE_INIT("module_load");
+    hipModule_t m = nullptr;
+    HIP_TRY(hipModuleLoadData(&m, image));
+    std::lock_guard<std::mutex> lock(g_module_mu);
+    g_modules[(void *)m] = 1;
+    *module = (void *)m;
+    return 0;
+}
+
+int miw_module_get_kernel(void *module, const char *name, void **kernel)
+{
+    if (!module || !name || !kernel) return fail(MIW_ERR_NULL_POINTER, "module_get_kernel: null argument");
+    *kernel = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_module_mu);
+        if (!g_modules.count(module)) return fail(MIW_ERR_NOT_FOUND, "module_get_kernel: not a module of miw_module_load");
+    }
+    REQUIRE_INIT("module_get_kernel");
+    hipFunction_t f = nullptr;
+    hipError_t e = hipModuleGetFunction(&f, (hipModule_t)module, name);
+    if (e == hipErrorNotFound) return fail(MIW_ERR_NOT_FOUND, "module_get_kernel: no kernel named '%s' in the module", name);
+    HIP_TRY(e);
+    std::lock_guard<std::mutex> lock(g_module_mu);
+    g_module_kernels[(void *)f] = module;
+    *kernel = (void *)f;
+    return 0;
+}
+
+int miw_module_unload(void *module)
+{
+    if (!module) return 0;
+    {
+        std::lock_guard<std::mutex> lock(g_module_mu);
+        if (!g_modules.count(module)) return fail(MIW_ERR_NOT_FOUND, "module_unload: not a module of miw_module_load");
+        for (auto it = g_module_kernels.begin(); it != g_module_kernels.end();)
+            it = it->second == module ? g_module_kernels.erase(it) : std::next(it);
+        g_modules.erase(module);
+    }
+    REQUIRE_INIT("module_unload");
+    HIP_TRY(hipModuleUnload((hipModule_t)module));
     return 0;
 }
 
 int miw_launch(void *kernel, const unsigned grid[3], const unsigned block[3], unsigned shmem, void *stream, void **args)
 {
     if (!kernel || !grid || !block) return fail(MIW_ERR_NULL_POINTER, "launch: null argument");
+    if (is_module_kernel(kernel)) {
+        const unsigned long nthreads = (unsigned long)block[0] * block[1] * block[2];
+        if (nthreads == 0 || (unsigned long)grid[0] * grid[1] * grid[2] == 0)
+            return fail(MIW_ERR_INVALID_VALUE, "launch: empty grid or block");
+        if (shmem > 64u * 1024u)
+            return fail(MIW_ERR_UNSUPPORTED, "launch: kernels of loaded code objects get at most 64 KiB of dynamic LDS (%u asked)", shmem);
+        REQUIRE_INIT("launch");
+        hipFunction_t f = (hipFunction_t)kernel;
+        int max_threads = 0;
+        HIP_TRY(hipFuncGetAttribute(&max_threads, HIP_FUNC_ATTRIBUTE_MAX_THREADS_PER_BLOCK, f));
+        if (nthreads > (unsigned long)max_threads)
+            return fail((int)hipErrorInvalidConfiguration, "launch: %lu threads per block exceed the kernel's maximum %d",
+                        nthreads, max_threads);
+        HIP_TRY(hipModuleLaunchKernel(f, grid[0], grid[1], grid[2], block[0], block[1], block[2], shmem, as_stream(stream), args,
+                                      nullptr));
+        return 0;
+    }
     bool known = false;
     for (auto &k : registry()) known = known || (void *)k.fn == kernel;
     if (!known) return fail(MIW_ERR_NOT_FOUND, "launch: not a kernel of this library");

@@ -3,7 +3,7 @@
 // directly with the fragment API (one wavefront per 16x16 output tile, the
 // "D of one mma is C of the next" chain of docs/src/device/wmma.md:51-52).
 #include "kernels.hpp"
-#include "wmma_fragment.hpp"
+#include "miwmma_fragment.hpp"
 
 namespace miw {
 

@@ -75,11 +75,14 @@ def cudaconvert(arg):
 class HostKernel:
     """A kernel of the library, callable with launch keywords (src/execution.jl:205-219)."""
 
-    def __init__(self, name):
-        p = ctypes.c_void_p()
-        _lib.check(_lib.load().miw_kernel_lookup(name.encode(), ctypes.byref(p)))
+    def __init__(self, name, fun=None, module=None):
+        if fun is None:
+            p = ctypes.c_void_p()
+            _lib.check(_lib.load().miw_kernel_lookup(name.encode(), ctypes.byref(p)))
+            fun = p.value
         self.name = name
-        self.fun = p.value
+        self.fun = fun
+        self.module = module      # keeps a loaded code object alive as long as its kernels
 
     def _attrs(self):
         a = _lib.KernelAttributes()
@@ -114,6 +117,35 @@ class HostKernel:
         grid = (ctypes.c_uint * 3)(*_dim3(blocks))
         block = (ctypes.c_uint * 3)(*_dim3(threads))
         _lib.check(_lib.load().miw_launch(self.fun, grid, block, int(shmem), _stream_handle(stream), slots))
+
+
+class Module:
+    """A code object of the caller's own, compiled ahead of time for gfx950 (hipcc --genco): the
+    CuModule(image) / CuFunction(mod, name) pair that cufunction ends in (src/execution.jl:300-342)."""
+
+    def __init__(self, image):
+        if isinstance(image, str):
+            with open(image, "rb") as f:
+                image = f.read()
+        p = ctypes.c_void_p()
+        _lib.check(_lib.load().miw_module_load(image, len(image), ctypes.byref(p)))
+        self.handle = p.value
+
+    def kernel(self, name):
+        p = ctypes.c_void_p()
+        _lib.check(_lib.load().miw_module_get_kernel(self.handle, name.encode(), ctypes.byref(p)))
+        return HostKernel(name, fun=p.value, module=self)
+
+    def unload(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            _lib.check(_lib.load().miw_module_unload(h))
+
+    def __del__(self):
+        try:
+            self.unload()
+        except Exception:
+            pass
 
 
 def kernel_names():

@@ -280,6 +280,17 @@ int miw_kernel_occupancy(void *kernel, size_t dynamic_shmem, int *min_grid, int 
 int miw_launch(void *kernel, const unsigned grid[3], const unsigned block[3], unsigned shmem,
                void *stream, void **args);
 
+/* Kernels of the caller's own: what cufunction ends in, CuModule(image) and CuFunction(mod, name)
+   (src/execution.jl:300-342), for code objects compiled ahead of time (hipcc --genco
+   --offload-arch=gfx950; the device-side fragment API is include/miwmma_fragment.hpp).  `image` is
+   a host buffer holding an ELF code object or a clang offload bundle; it may be released after the
+   call.  Kernels obtained from a module work with miw_kernel_attributes_get,
+   miw_kernel_occupancy and miw_launch (at most 64 KiB of dynamic LDS) until the module is
+   unloaded; unloading while one of its kernels is still running is undefined. */
+int miw_module_load(const void *image, size_t bytes, void **module);
+int miw_module_get_kernel(void *module, const char *name, void **kernel);
+int miw_module_unload(void *module);
+
 #ifdef __cplusplus
 }
 #endif

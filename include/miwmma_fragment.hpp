@@ -1,4 +1,7 @@
-// Device-side WMMA fragment API for gfx950 (wave64, MFMA).
+// Device-side WMMA fragment API for gfx950 (wave64, MFMA): include it from a HIP kernel of your
+// own (hipcc --offload-arch=gfx950 -I<this directory>), build the kernel into a code object
+// (--genco) and run it through miw_module_load / miw_module_get_kernel / miw_launch, or link it
+// into a HIP program directly.  The kernels inside libmiwmma.so are written with the same header.
 //
 // Counterpart of CUDAnative.jl's WMMA module (src/device/cuda/wmma.jl):
 //   Config{M,N,K,d_type}            :394      -> miw::config<M,N,K,D>

@@ -296,3 +296,20 @@ def test_tile_counts_that_overflow_the_grid_are_refused(miw):
     # (too many) and 2^21 tiles of 256 x 256 with 512 (fine)
     d = G.make_desc(1 << 19, 1 << 18, 64)
     assert not G.variant_supports(d, 8) and G.variant_supports(d, 1)
+
+
+def test_module_entries_check_their_arguments_without_a_device(miw):
+    L = miw._lib
+    lib = L.load()
+    p = ctypes.c_void_p()
+    assert lib.miw_module_load(b"x" * 100, 100, ctypes.byref(p)) == L.ERR_INVALID_VALUE and not p.value
+    assert lib.miw_module_load(None, 0, ctypes.byref(p)) == L.ERR_NULL_POINTER
+    assert lib.miw_module_load(b"\x7fELF" + b"\0" * 10, 14, ctypes.byref(p)) == L.ERR_INVALID_VALUE      # shorter than an ELF header
+    assert lib.miw_module_get_kernel(None, b"k", ctypes.byref(p)) == L.ERR_NULL_POINTER
+    assert lib.miw_module_get_kernel(ctypes.c_void_p(64), b"k", ctypes.byref(p)) == L.ERR_NOT_FOUND
+    assert lib.miw_module_unload(ctypes.c_void_p(64)) == L.ERR_NOT_FOUND and lib.miw_module_unload(None) == 0
+    # the example code object is built with the library and is a gfx950 ELF
+    path = os.path.join(ROOT, "cudanative.jl_amd", "examples", "user_kernel.hsaco")
+    if os.path.exists(path):
+        head = open(path, "rb").read(64)
+        assert head[:4] == b"\x7fELF" or head.startswith(b"__CLANG_OFFLOAD_BUNDLE__")
