@@ -7,7 +7,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmiwmma.so")
+# MIWMMA_LIB names another build of the library (a measurement build made by build.py --define ... --output)
+LIB_PATH = os.environ.get("MIWMMA_LIB") or os.path.join(HERE, "libmiwmma.so")
 
 ROW_MAJOR, COL_MAJOR = 0, 1
 F16, F32 = 0, 1
@@ -129,6 +130,7 @@ SIGNATURES = {
     "miw_gemm": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _vp]),
     "miw_gemm_variant_count": (_i, []),
     "miw_gemm_variant_info_get": (_i, [_i, ctypes.POINTER(GemmVariantInfo)]),
+    "miw_build_id": (ctypes.c_char_p, []),
     "miw_gemm_variant_supports": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(_i)]),
     "miw_gemm_pick_variant": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
     "miw_gemm_acc_chunk": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),

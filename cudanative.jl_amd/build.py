@@ -25,6 +25,20 @@ FLAGS = [
 ]
 
 
+def source_id():
+    """Hash of every file the library is compiled from; the library carries the one it was built with
+    (miw_build_id), so a stale binary can be told from a current one."""
+    import hashlib
+    h = hashlib.sha256()
+    files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".hpp"))]
+    files += [os.path.join(INCLUDE, f) for f in sorted(os.listdir(INCLUDE)) if f.endswith((".h", ".hpp"))]
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def hipcc():
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -32,13 +46,19 @@ def hipcc():
     return exe
 
 
-def build(verbose=False, extra_flags=()):
-    """Compile every kernel translation unit and link libmiwmma.so."""
+def build(verbose=False, extra_flags=(), output=None):
+    """Compile every kernel translation unit and link libmiwmma.so (or `output`: a measurement
+    build with extra -D switches goes to a path of its own, objects in a directory beside it, and
+    never replaces the library)."""
+    if output is not None:
+        return _build_variant(verbose, list(extra_flags), os.path.abspath(output))
     objs = []
     procs = []
+    build_id = source_id()
     for src in SOURCES:
         obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-        cmd = [hipcc(), *FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        ident = ['-DMIW_BUILD_ID="%s"' % build_id] if src == "capi.hip" else []
+        cmd = [hipcc(), *FLAGS, *extra_flags, *ident, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -58,6 +78,27 @@ def build(verbose=False, extra_flags=()):
     return LIB
 
 
+def _build_variant(verbose, extra_flags, output):
+    objdir = output + ".objs"
+    os.makedirs(objdir, exist_ok=True)
+    procs, objs = [], []
+    for src in SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        ident = ['-DMIW_BUILD_ID="%s+%s"' % (source_id(), " ".join(extra_flags))] if src == "capi.hip" else []
+        cmd = [hipcc(), *FLAGS, *extra_flags, *ident, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+    for cmd, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd), out))
+    subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", output, *objs])
+    shutil.rmtree(objdir, ignore_errors=True)
+    return output
+
+
 def build_example(verbose=False):
     """The user-kernel example as a gfx950 code object, for miw_module_load."""
     cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++20", "--genco", "-I" + INCLUDE,
@@ -72,4 +113,19 @@ def build_example(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build(verbose="-q" not in sys.argv))
+    # python build.py [-q] [--define NAME[=VALUE]]... [--output PATH]
+    # --define adds -DNAME=VALUE to every translation unit (the measurement switches MIW_PP_ABLATE and
+    # MIW_PP_TS); with it an --output path other than the library's own is required.
+    argv = sys.argv[1:]
+    defines, output = [], None
+    while "--define" in argv:
+        i = argv.index("--define")
+        defines.append("-D" + argv[i + 1])
+        del argv[i:i + 2]
+    if "--output" in argv:
+        i = argv.index("--output")
+        output = argv[i + 1]
+        del argv[i:i + 2]
+    if defines and output is None:
+        sys.exit("build.py: --define needs --output (a measurement build must not replace libmiwmma.so)")
+    print(build(verbose="-q" not in argv, extra_flags=defines, output=output))

@@ -253,6 +253,11 @@ extern "C" {
 
 const char *miw_last_error(void) { return g_err; }
 
+#ifndef MIW_BUILD_ID
+#define MIW_BUILD_ID "unknown"
+#endif
+const char *miw_build_id(void) { return MIW_BUILD_ID; }
+
 int miw_init(int device)
 {
     int n = 0;

@@ -44,6 +44,8 @@ Base.showerror(io::IO, e::MIWError) = print(io, "miwmma error ", e.code, ": ", e
 
 last_error() = unsafe_string(ccall((:miw_last_error, libmiwmma), Cstring, ()))
 check(rc::Cint) = rc == 0 ? nothing : throw(MIWError(rc, last_error()))
+"Hash of the sources the loaded library was built from."
+build_id() = unsafe_string(ccall((:miw_build_id, libmiwmma), Cstring, ()))
 
 const hipErrorOutOfMemory = Cint(2)
 

@@ -70,6 +70,10 @@ int miw_init(int device);
 /* Message for the last failing call on this thread ("" if none). */
 const char *miw_last_error(void);
 
+/* Hash of the sources this library was compiled from (16 hex digits; the build recipe computes
+   it), so that tests and benchmarks can tell a stale binary from a current one. */
+const char *miw_build_id(void);
+
 typedef struct miw_device_info {
     char name[128];
     char arch[64];

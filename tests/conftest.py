@@ -15,11 +15,22 @@ def load_package():
     name = "cudanative_jl_amd"
     if name in sys.modules:
         return sys.modules[name]
-    if not os.path.exists(os.path.join(PKG_DIR, "libmiwmma.so")):
-        # nothing built yet: build once (hipcc cross-compiles without a GPU)
-        spec_b = importlib.util.spec_from_file_location("_miw_build", os.path.join(PKG_DIR, "build.py"))
-        b = importlib.util.module_from_spec(spec_b)
-        spec_b.loader.exec_module(b)
+    spec_b = importlib.util.spec_from_file_location("_miw_build", os.path.join(PKG_DIR, "build.py"))
+    b = importlib.util.module_from_spec(spec_b)
+    spec_b.loader.exec_module(b)
+    lib_path = os.path.join(PKG_DIR, "libmiwmma.so")
+    stale = False
+    if os.path.exists(lib_path):
+        # the library carries the hash of the sources it was built from
+        import ctypes
+        probe = ctypes.CDLL(lib_path)
+        try:
+            probe.miw_build_id.restype = ctypes.c_char_p
+            stale = probe.miw_build_id().decode() != b.source_id()
+        except AttributeError:      # a library from before the hash existed
+            stale = True
+    if stale or not os.path.exists(lib_path):
+        # nothing built yet, or built from other sources: build once (hipcc cross-compiles without a GPU)
         b.build()
     spec = importlib.util.spec_from_file_location(name, os.path.join(PKG_DIR, "__init__.py"),
                                                   submodule_search_locations=[PKG_DIR])
@@ -27,6 +38,14 @@ def load_package():
     sys.modules[name] = mod
     spec.loader.exec_module(mod)
     return mod
+
+
+def pytest_report_header(config):
+    try:
+        m = load_package()
+        return "libmiwmma build id: %s" % m._lib.load().miw_build_id().decode()
+    except Exception as e:  # noqa: BLE001
+        return "libmiwmma not loadable: %s" % e
 
 
 def pytest_configure(config):
