@@ -81,6 +81,36 @@ def cpu_baseline(orc, M, N, K, batch, budget_s=20.0):
     }
 
 
+def library_reference():
+    """torch.matmul on 4096^3 Float16 matrices (Float16 output, no C operand; torch.addmm for a Float16 C),
+    timed like the benchmark: spin-up, then 200 back-to-back launches between two synchronisations."""
+    import torch
+    n = 4096
+    a = (torch.rand(n, n, device="cuda") * 2 - 1).half()
+    b = (torch.rand(n, n, device="cuda") * 2 - 1).half()
+    c = (torch.rand(n, n, device="cuda") * 2 - 1).half()
+    # torch matrices are row-major: X.t() is the column-major operand
+    cases = {"A col-major, B col-major": lambda: torch.matmul(b, a),        # D^T = B^T A^T on the row-major views
+             "A row-major, B col-major": lambda: torch.matmul(a, b.t()),
+             "A col-major, B row-major": lambda: torch.matmul(a.t(), b),
+             "A row-major, B row-major": lambda: torch.matmul(a, b),
+             "A row-major, B row-major, + Float16 C (addmm)": lambda: torch.addmm(c, a, b)}
+    out = {}
+    for name, fn in cases.items():
+        t_spin = time.perf_counter()
+        while time.perf_counter() - t_spin < 0.3:
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            fn()
+        torch.cuda.synchronize()
+        t = (time.perf_counter() - t0) / 200
+        out[name] = {"us": t * 1e6, "tflops": 2.0 * n ** 3 / t / 1e12}
+    print(json.dumps({"library_reference": "torch.matmul Float16 4096^3 (torch %s)" % torch.__version__, "results": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -93,6 +123,11 @@ def main():
     ap.add_argument("--rotate", type=int, default=1, help="cycle the timed launches through N copies of the operands")
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--a-layout", choices=("col", "row"), help="override the configuration's layout of A")
+    ap.add_argument("--b-layout", choices=("col", "row"), help="override the configuration's layout of B")
+    ap.add_argument("--library-reference", action="store_true",
+                    help="instead of this library, time the vendor GEMM (hipBLASLt / rocBLAS through torch.matmul) on "
+                         "4096^3 Float16 operands in the four operand layouts and print one line; a comparison aid")
     ap.add_argument("--operand-scale", type=float, default=1.0,
                     help="multiply A and B by this before rounding to Float16 (0: all-zero operands, which lift the "
                          "power cap off the matrix cores; a measurement aid, not the benchmark)")
@@ -110,6 +145,9 @@ def main():
               "(--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
 
+    if args.library_reference:
+        library_reference()
+        return
     from __graft_entry__ import load_package
     from oracle import oracle as orc
     m = load_package()
@@ -133,7 +171,10 @@ def main():
         return
     info = m.device_info()
     W, G = m.WMMA, m.GEMM
-    cfg = CONFIGS[args.config]
+    cfg = dict(CONFIGS[args.config])
+    if args.a_layout or args.b_layout:
+        cfg["a"], cfg["b"] = args.a_layout or cfg["a"], args.b_layout or cfg["b"]
+        cfg["workload"] += " [A %s-major, B %s-major]" % (cfg["a"], cfg["b"])
     M, N, K, batch = cfg["M"], cfg["N"], cfg["K"], cfg["batch"]
     half = cfg["half"]
     ct = np.float16 if half else np.float32
