@@ -37,11 +37,12 @@ namespace miw {
 #endif
 
 // Second measurement switch (off in every shipped build; gemm_kernels.hip must be compiled with it
-// too): with MIW_PP_TS the 64-k-cluster kernel records, per wavefront, the shader clock at kernel
+// too): with MIW_PP_TS the ping-pong kernels record, per wavefront, the shader clock at kernel
 // entry [0], after the prologue's loads have landed [1], at the middle of the loop [2], one pair
-// later [3], at the end of the loop [4], when the last store is issued [5] and when the stores have
-// drained [6], plus the 100 MHz wall clock at exit [7] and entry [8], into the buffer whose device
-// address the environment variable MIW_TS holds.
+// of k-steps later [3], at the end of the pairs that do not fold C [9], at the end of the loop [4],
+// when the last store is issued [5] and when the stores have drained [6], plus the 100 MHz wall
+// clock at exit [7] and entry [8], into the buffer whose device address the environment variable
+// MIW_TS holds (cudanative.jl_amd/timestamps.py sets it and prints the phases).
 #ifdef MIW_PP_TS
 #define MIW_PP_STAMP(i) { __builtin_amdgcn_sched_barrier(0); ts[i] = clock64(); __builtin_amdgcn_sched_barrier(0); }
 #else
@@ -142,6 +143,11 @@ void k_gemm_pp(tiled_params p)
     constexpr int ND = xop::PER_CLUSTER + yop::PER_CLUSTER;  // loads per thread and memory cluster
     static_assert(pp_fits(BI, BJ, XK, YK), "ring does not fit in LDS");
 
+#ifdef MIW_PP_TS
+    long long ts[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    ts[0] = clock64();
+    ts[8] = wall_clock64();
+#endif
     extern __shared__ __attribute__((aligned(128))) char smem[];
     MIW_LDS char *lds = (MIW_LDS char *)smem;
 
@@ -395,12 +401,18 @@ void k_gemm_pp(tiled_params p)
     };
     constexpr std::integral_constant<int, -1> no_fold{};
 
+    MIW_PP_STAMP(1)
     if (late_group) __builtin_amdgcn_s_barrier();
     const int NPM = fold_c ? NP - NFOLD / 2 : NP;
     for (int pr = 0; pr < NPM; pr++) {
+#ifdef MIW_PP_TS
+        if (pr == NPM / 2) MIW_PP_STAMP(2)
+        if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
+#endif
         step(std::integral_constant<int, 0>{}, no_fold);
         step(std::integral_constant<int, 1>{}, no_fold);
     }
+    MIW_PP_STAMP(9)
     if constexpr (CAN_FOLD) {
         if (fold_c) {
             [&]<int... G>(std::integer_sequence<int, G...>) {
@@ -418,6 +430,7 @@ void k_gemm_pp(tiled_params p)
         }
     }
     if (!late_group) __builtin_amdgcn_s_barrier();
+    MIW_PP_STAMP(4)
 
     // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
     auto read_c = [&](int a, int b, bool trans) -> float4_t {
@@ -459,6 +472,14 @@ void k_gemm_pp(tiled_params p)
     if (!p.use_c || fold_c) epilogue(false, false);
     else if (p.c_trans) epilogue(true, true);
     else epilogue(true, false);
+#ifdef MIW_PP_TS
+    MIW_PP_STAMP(5)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    MIW_PP_STAMP(6)
+    ts[7] = wall_clock64();
+    if (p.ts && lane == 0)
+        for (int i = 0; i < 10; i++) p.ts[((long)(blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 10 + i] = ts[i];
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -473,8 +494,7 @@ void k_gemm_pp(tiled_params p)
 //
 // fp16 accumulation rounds the running sums to Float16 once per slot (64 k-values): a tile is
 // rounded two MFMAs after its last MFMA of the pair, inside the compute cluster (the memory
-// cluster is the longer of the two: the LDS serves 128 bytes a clock and is the unit these tiles
-// keep busiest).  The C operand is requested before anything else, converted once the prologue's
+// cluster is the longer of the two at these tiles: it takes about 530 cycles whatever it holds).  The C operand is requested before anything else, converted once the prologue's
 // loads have landed and added at the first rounding: acc = half(half(beta * C) + sum of the first
 // 64 k-values), so that its latency hides behind the prologue.
 template <int BI, int BJ, int WI, int WJ, int NSLOT, bool XK, bool YK, class CT, class DT, bool F16ACC>
