@@ -150,8 +150,10 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
 #endif
     const void *fn = pick_kernel(i, xk, yk, c_type, d_type, f16acc);
     if (!fn) return hipErrorInvalidValue;
+    // (the 64-k ping-pong kernels stage a Float16 C tile beside the ring where both fit)
+    const int c_stage = v.kind == KIND_PINGPONG64 && f16acc && v.lds_bytes + v.bm * v.bn * 2 <= 160 * 1024 ? v.bm * v.bn * 2 : 0;
     const int lds_bytes = v.kind == KIND_PINGPONG32 ? pp_lds(v.bm, v.bn, xk, yk)
-                          : v.kind != KIND_PIPELINED ? v.lds_bytes
+                          : v.kind != KIND_PIPELINED ? v.lds_bytes + c_stage
                                                      : v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
     hipError_t e = allow_dynamic_lds(fn, lds_bytes);
     if (e != hipSuccess) return e;

@@ -613,9 +613,31 @@ void k_gemm_pp64(tiled_params p)
     // before the prologue's wait (a conversion here would make the compiler wait for the loads
     // before the first direct-to-LDS load is issued).  C laid out as D: the lane's four halves in two
     // registers; C stored across D: one zero-extended half per register.
+    //
+    // Where LDS has room for the workgroup's whole tile of C beside the ring (128 x 128: 32 KiB), a C laid
+    // out as D comes through LDS instead: the accumulator layout reads 32 contiguous bytes per column
+    // and instruction, which costs the 128 x 128 kernel 6000 cycles of prologue, whereas direct-to-LDS
+    // loads fetch whole 256-byte columns (16 lanes per column).  Chunk (column j, 16-byte piece c) sits at
+    // chunk index j * 16 + (c ^ (j & 15)), so that the 16 lanes that later read 16 columns at one row
+    // offset hit 16 different 16-byte slots.
+    constexpr bool C_STAGE_FITS = F16ACC && NSLOT * SLOT + BI * BJ * 2 <= 160 * 1024 && (BI * 2) % 256 == 0;
+    constexpr int C_STAGE = NSLOT * SLOT;                         // byte offset of the staged tile
+    constexpr int C_CHUNKS_PER_COL = BI * 2 / 16, NLC = C_STAGE_FITS ? BI * BJ * 2 / 16 / NT : 0;
+    const bool c_staged = C_STAGE_FITS && p.use_c && !p.c_trans && p.ldc < (1l << 22);  // (32-bit lane offsets)
+    if constexpr (C_STAGE_FITS) {
+        if (c_staged) {
+            const char *ctile = (const char *)(C + (long)j0 * p.ldc + i0);
+#pragma unroll
+            for (int n = 0; n < NLC; n++) {
+                const int g = n * NT + tid;
+                const int j = g / C_CHUNKS_PER_COL, c = (g % C_CHUNKS_PER_COL) ^ (j & 15);
+                lds_dma16(ctile, (unsigned)(j * (int)p.ldc * 2 + c * 16), wave_dst + (unsigned)(C_STAGE + n * NT * 16));
+            }
+        }
+    }
     unsigned craw[F16ACC ? TI : 1][F16ACC ? TJ : 1][4];
     if constexpr (F16ACC) {
-        if (p.use_c) {
+        if (p.use_c && !c_staged) {
             auto fetch = [&]<bool TRANS>(std::bool_constant<TRANS>) {
 #pragma unroll
                 for (int a = 0; a < TI; a++)
@@ -664,6 +686,19 @@ void k_gemm_pp64(tiled_params p)
             for (int a = 0; a < TI; a++)
 #pragma unroll
                 for (int b = 0; b < TJ; b++) cinit[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+        } else if (c_staged) {
+            if constexpr (C_STAGE_FITS) {
+#pragma unroll
+                for (int a = 0; a < TI; a++)
+#pragma unroll
+                    for (int b = 0; b < TJ; b++) {
+                        const int j = wj * WTJ + 16 * b + r, i = wi * WTI + 16 * a + 4 * q;
+                        const int at = C_STAGE + (j * C_CHUNKS_PER_COL + ((i >> 3) ^ (j & 15))) * 16 + (i & 7) * 2;
+                        const half4_t h = *(MIW_LDS const half4_t *)(lds + at);
+#pragma unroll
+                        for (int v = 0; v < 4; v++) cinit[a][b][v] = round_through_half(p.beta * (float)h[v]);
+                    }
+            }
         } else if (p.c_trans) {
             convert(std::true_type{});
         } else {
