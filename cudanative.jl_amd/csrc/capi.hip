@@ -1015,7 +1015,10 @@ int miw_module_get_kernel(void *module, const char *name, void **kernel)
     REQUIRE_INIT("module_get_kernel");
     hipFunction_t f = nullptr;
     hipError_t e = hipModuleGetFunction(&f, (hipModule_t)module, name);
-    if (e == hipErrorNotFound) return fail(MIW_ERR_NOT_FOUND, "module_get_kernel: no kernel named '%s' in the module", name);
+    if (e == hipErrorNotFound) {
+        (void)hipGetLastError();  // the runtime keeps the failure as its "last error": clear it, or the next launch would report it
+        return fail(MIW_ERR_NOT_FOUND, "module_get_kernel: no kernel named '%s' in the module", name);
+    }
     HIP_TRY(e);
     std::lock_guard<std::mutex> lock(g_module_mu);
     g_module_kernels[(void *)f] = module;

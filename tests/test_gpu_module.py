@@ -87,6 +87,9 @@ def test_module_errors(gpu):
     with pytest.raises(gpu.MIWError) as e:
         mod.kernel("no_such_kernel")
     assert e.value.code == L.ERR_NOT_FOUND
+    # the failed lookup must not linger as the runtime's "last error": the next launches succeed
+    frag = gpu.WMMA.fill_c(np.float32(3.0), gpu.WMMA.Config[16, 16, 16, F32])
+    assert np.all(np.asarray(frag.x) == 3.0)
     k = mod.kernel("user_mac")
     u3 = (ctypes.c_uint * 3)
     assert lib.miw_launch(k.fun, u3(1, 1, 1), u3(64, 1, 1), 100 * 1024, None, None) == L.ERR_UNSUPPORTED
