@@ -163,7 +163,9 @@ bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f
     if (p.use_c && (p.ldc % cper || p.sc % cper)) return false;
     // 32-bit offsets inside one operand tile
     if (p.lda * 256 >= (1l << 31) || p.ldb * 256 >= (1l << 31)) return false;
-    if (f16acc && (!miw::tiled_supports_f16acc(i) || p.alpha != 1.0f ||
+    // fp16 accumulation: the pipelined kernels round their MFMA accumulators in place, which needs
+    // alpha == 1; the 64-k ping-pong kernels keep the running sum apart and take any alpha
+    if (f16acc && (!miw::tiled_supports_f16acc(i) || (p.alpha != 1.0f && v.kind != miw::KIND_PINGPONG64) ||
                    (acc_chunk != 0 && acc_chunk != miw::tiled_f16acc_chunk())))
         return false;
     return true;
@@ -234,7 +236,7 @@ int check_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, i
                     "dimensions, a tile count that fits the launch grid, and (ping-pong kernels) at most one operand "
                     "with k contiguous%s",
                     variant, miw::tiled_variant_at(variant - 1).name,
-                    f16acc ? ", alpha == 1, its own acc_chunk, and accumulators that fit in VGPRs" : "");
+                    f16acc ? ", alpha == 1 (the 64-k ping-pong kernels take any alpha), its own acc_chunk, and accumulators that fit in VGPRs" : "");
     }
     *variant_out = variant;
     return 0;

@@ -492,11 +492,12 @@ void k_gemm_pp(tiled_params p)
 // two barriers that follow publish it before anyone reads it.  Both operand kinds use the slot
 // layouts, loaders and fragment readers of gemm_tiled.hpp.
 //
-// fp16 accumulation rounds the running sums to Float16 once per slot (64 k-values): a tile is
-// rounded two MFMAs after its last MFMA of the pair, inside the compute cluster (the memory
-// cluster is the longer of the two at these tiles: it takes about 530 cycles whatever it holds).  The C operand is requested before anything else, converted once the prologue's
-// loads have landed and added at the first rounding: acc = half(half(beta * C) + sum of the first
-// 64 k-values), so that its latency hides behind the prologue.
+// fp16 accumulation rounds once per slot (64 k-values), two MFMAs after a tile's last MFMA of the pair,
+// inside the compute cluster; with alpha == 1 the MFMAs accumulate onto the rounded sum in place,
+// otherwise the running sum is kept beside accumulators that restart from zero in every slot:
+// run = half(run + alpha * slot sum) (the memory
+// cluster is the longer of the two at these tiles: it takes about 530 cycles whatever it holds).  The running sum starts as half(beta * C): C is requested before anything else and
+// converted once the prologue's loads have landed.
 template <int BI, int BJ, int WI, int WJ, int NSLOT, bool XK, bool YK, class CT, class DT, bool F16ACC>
 __global__ __launch_bounds__(WI *WJ * 64) __attribute__((amdgpu_waves_per_eu(2)))
 void k_gemm_pp64(tiled_params p)
@@ -711,16 +712,25 @@ void k_gemm_pp64(tiled_params p)
         [&]<int... U>(std::integer_sequence<int, U...>) { ((fx[0][U] = fx[1][U] = xr.template read<U, 0>(lds)), ...); }(std::make_integer_sequence<int, TI>{});
         [&]<int... U>(std::integer_sequence<int, U...>) { ((fy[0][U] = fy[1][U] = yr.template read<U, 0>(lds + XBYTES)), ...); }(std::make_integer_sequence<int, TJ>{});
     }
-    // Rounding of the tile MFMA number m of a k-step works on.  FIRST: the pair's sums meet the C operand here.
-    auto round_tile = [&]<bool FIRST>(int m, std::bool_constant<FIRST>) {
+    // fp16 accumulation, for the tile MFMA number m of a k-step works on.
+    // RMODE 1, 2 (alpha == 1): the MFMAs accumulate onto the rounded running sum, which is rounded in
+    //     place once per slot; in the first slot (2) the sum meets half(beta * C) here.
+    // RMODE 3 (any alpha): `cinit` is the running sum (a Float16 value held as Float32), the MFMA
+    //     accumulators restart from zero in every slot and run = half(run + alpha * slot sum).
+    auto round_tile = [&]<int RMODE>(int m, std::integral_constant<int, RMODE>) {
         const int a = m / TJ, b = serpentine_column(m, TJ);
         float4_t v = acc[a][b];
-        if constexpr (FIRST) {
+        if constexpr (RMODE == 2) {
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] += cinit[a][b][e];
         }
+        if constexpr (RMODE == 3) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.alpha, v[e], cinit[a][b][e]);
+        }
         half4_t h = __builtin_convertvector(v, half4_t);
-        acc[a][b] = __builtin_convertvector(h, float4_t);
+        if constexpr (RMODE == 3) cinit[a][b] = __builtin_convertvector(h, float4_t);
+        else acc[a][b] = __builtin_convertvector(h, float4_t);
     };
     // Fragment unit U of a memory cluster (step 0: the TI x-fragments, then the TJ y-fragments; then
     // step 1), preceded by the direct-to-LDS loads that go out before it (load n before unit
@@ -755,8 +765,8 @@ void k_gemm_pp64(tiled_params p)
         rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
         __builtin_amdgcn_sched_barrier(0);
     };
-    // RMODE 0: fp32 sums; 1: round every tile to Float16 ROUND_LAG MFMAs after its last MFMA of the
-    // pair; 2: the same for the first pair, which adds the C operand.
+    // RMODE 0: fp32 sums over all of K; 1-3 (fp16 accumulation, see round_tile): each tile is rounded
+    // ROUND_LAG MFMAs after its last MFMA of the pair.
     constexpr int ROUND_LAG = 2;
     auto compute_cluster = [&]<int RMODE>(std::integral_constant<int, RMODE>) {
         __builtin_amdgcn_sched_barrier(0);
@@ -766,14 +776,17 @@ void k_gemm_pp64(tiled_params p)
             for (int m = 0; m < NTILE; m++) {
                 // serpentine order: every MFMA changes exactly one of its two operand fragments
                 const int a = m / TJ, b = serpentine_column(m, TJ);
-                if constexpr (!(MIW_PP_ABLATE & 4)) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], acc[a][b], 0, 0, 0);
+                if constexpr (!(MIW_PP_ABLATE & 4)) {
+                    if (RMODE == 3 && h == 0) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    else acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], acc[a][b], 0, 0, 0);
+                }
                 if constexpr (RMODE != 0)
-                    if (h == 1 && m >= ROUND_LAG) round_tile(m - ROUND_LAG, std::bool_constant<RMODE == 2>{});
+                    if (h == 1 && m >= ROUND_LAG) round_tile(m - ROUND_LAG, std::integral_constant<int, RMODE>{});
                 __builtin_amdgcn_sched_barrier(0);
             }
         if constexpr (RMODE != 0)
 #pragma unroll
-            for (int m = NTILE > ROUND_LAG ? NTILE - ROUND_LAG : 0; m < NTILE; m++) round_tile(m, std::bool_constant<RMODE == 2>{});
+            for (int m = NTILE > ROUND_LAG ? NTILE - ROUND_LAG : 0; m < NTILE; m++) round_tile(m, std::integral_constant<int, RMODE>{});
     };
 
     // Folding C (Float32 C laid out as D, alpha == 1): CPT MFMA tiles per cluster over the last
@@ -838,13 +851,19 @@ void k_gemm_pp64(tiled_params p)
     MIW_PP_STAMP(1)
     if (late_group) __builtin_amdgcn_s_barrier();
     const int NPM = fold_c ? NP - NFOLD : NP;
-    if (NPM > 0) pair(no_fold, std::integral_constant<int, F16ACC ? 2 : 0>{});
-    for (int pr = 1; pr < NPM; pr++) {
+    const bool separate_sum = F16ACC && p.alpha != 1.0f;
+    if (separate_sum) {
+        if constexpr (F16ACC)
+            for (int pr = 0; pr < NPM; pr++) pair(no_fold, std::integral_constant<int, 3>{});
+    } else {
+        if (NPM > 0) pair(no_fold, std::integral_constant<int, F16ACC ? 2 : 0>{});
+        for (int pr = 1; pr < NPM; pr++) {
 #ifdef MIW_PP_TS
-        if (pr == NPM / 2) MIW_PP_STAMP(2)
-        if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
+            if (pr == NPM / 2) MIW_PP_STAMP(2)
+            if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
 #endif
-        pair(no_fold, std::integral_constant<int, F16ACC ? 1 : 0>{});
+            pair(no_fold, std::integral_constant<int, F16ACC ? 1 : 0>{});
+        }
     }
     MIW_PP_STAMP(9)
     if constexpr (CAN_FOLD) {
@@ -871,7 +890,7 @@ void k_gemm_pp64(tiled_params p)
         for (int b = 0; b < TJ; b++)
 #pragma unroll
             for (int a = 0; a < TI; a++) {
-                float4_t v = acc[a][b];
+                float4_t v = separate_sum ? cinit[a][b] : acc[a][b];
                 if constexpr (!F16ACC) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) v[e] *= p.alpha;

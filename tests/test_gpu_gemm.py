@@ -387,7 +387,8 @@ def test_f16acc_exact_on_integers_all_variants(gpu, orc):
 
 
 def test_f16acc_alpha_beta(gpu, orc):
-    # alpha != 1 is served by the fragment-op kernel (rounding every 16); beta scales the initial accumulator
+    # alpha != 1 on a shape no LDS tile with a separate running sum divides: served by the fragment-op kernel
+    # (rounding every 16); beta scales the initial accumulator
     g = orc.GemmDesc(M=64, N=64, K=128, c_type=orc.F16, d_type=orc.F16, alpha=0.5, beta=2.0)
     A, B, C = _inputs(orc, g, 81, lo=-0.5, hi=0.5, clo=-0.1, chi=0.1)
     desc = gpu.GEMM.make_desc(64, 64, 128, c_type=F16, d_type=F16, acc_type=F16, alpha=0.5, beta=2.0)
@@ -395,8 +396,31 @@ def test_f16acc_alpha_beta(gpu, orc):
     D = _run(gpu, orc, g, A, B, C, acc_type=F16)
     model = orc.gemm_f16acc(g, 16, A, B, C)
     _assert_matches_model(D, model)
-    with pytest.raises(gpu.MIWError):                     # a tiled variant cannot honour alpha != 1 in fp16 accumulate
+    with pytest.raises(gpu.MIWError):                     # the pipelined tiles round in place: alpha must be 1
         _run(gpu, orc, g, A, B, C, acc_type=F16, variant=[v["id"] for v in _variants(gpu) if v["name"] == "tile64x64_w2x2"][0])
+
+
+@pytest.mark.parametrize("name,M,N", [("tile128x128_pingpong", 256, 128), ("tile256x128_pingpong", 256, 256),
+                                      ("tile128x256_pingpong", 128, 512)])
+def test_f16acc_any_alpha_on_the_64k_pingpong_kernels(gpu, orc, name, M, N):
+    """run = half(run + alpha * slot sum) with the running sum kept apart from the MFMA accumulators: exact
+    against the chunked model on quarter-integers (alpha a power of two), close to it on uniform data,
+    for C laid out as D (through LDS where it fits), across D, and absent."""
+    v = [x["id"] for x in _variants(gpu) if x["name"] == name][0]
+    for alpha, beta, cl, use_c in ((0.5, 2.0, orc.COL, 1), (-2.0, -1.0, orc.ROW, 1), (0.25, 1.0, orc.COL, 0)):
+        g = orc.GemmDesc(M=M, N=N, K=320, c_type=orc.F16, d_type=orc.F16, alpha=alpha, beta=beta, c_layout=cl,
+                         use_c=use_c, a_layout=orc.ROW, ldc=(M if cl == orc.COL else N) + 8)
+        A, B, C = _inputs(orc, g, 90, ints=True)
+        A, B = (A / 4).astype(F16), (B / 4).astype(F16)
+        desc = gpu.GEMM.make_desc(M, N, 320, c_type=F16, d_type=F16, acc_type=F16, alpha=alpha, beta=beta)
+        assert gpu.GEMM.acc_chunk(desc) == 64
+        D = _run(gpu, orc, g, A, B, C if use_c else None, variant=v, acc_type=F16)
+        assert np.array_equal(D, orc.gemm_f16acc(g, 64, A, B, C)), (name, alpha, beta, cl, use_c)
+    g = orc.GemmDesc(M=M, N=N, K=1024, c_type=orc.F16, d_type=orc.F16, alpha=0.75, beta=-1.5)
+    A, B, C = _inputs(orc, g, 91, lo=-0.5, hi=0.5, clo=-0.1, chi=0.1)
+    D = _run(gpu, orc, g, A, B, C, variant=v, acc_type=F16)
+    _assert_matches_model(D, orc.gemm_f16acc(g, 64, A, B, C))
+    assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TOL_F16ACC
 
 
 # ------------------------------------------------------------- benchmark configurations ---
