@@ -186,14 +186,27 @@ bool is_module_kernel(void *kernel)
 }
 int splitk_scratch(void **out);  // address of the current device's static split-K workspace (below)
 
-int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
+// Estimated duration of one launch of tiled variant i, in microseconds: a fixed cost per round of
+// workgroups, the C and D traffic at what the fabric sustains beside a running K loop, and the K
+// loop at the variant's measured pace (a CU that holds a queue of workgroups works through it at
+// the queued pace; below that, one workgroup cannot go faster than when it is alone on its CU).
+double estimate_us(int i, const miw::gemm_params &p, int c_type, int d_type)
 {
-    // Largest tile that still gives every CU a workgroup; else the one with most workgroups.
+    const miw::tiled_variant &v = miw::tiled_variant_at(i);
     const int cus = g_cu_count > 0 ? g_cu_count : 256;
     const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
-    int best = -1;
-    long best_wgs = -1;
-    // Tiles from large to small; of two kernels for one tile the ping-pong form goes first.
+    const long tiles = (I / v.bm) * (J / v.bn) * p.batch;
+    const long per_cu = (tiles + cus - 1) / cus;
+    const long rounds = (per_cu + v.occupancy - 1) / v.occupancy;
+    const double per_pair = std::max((double)v.us_pair_alone, (double)per_cu * v.us_pair_queued);
+    const double cd_bytes = (double)I * (double)J * (double)p.batch * (double)(dtype_size(d_type) + (p.use_c ? dtype_size(c_type) : 0));
+    return 4.5 * (double)rounds + cd_bytes / 5.5e6 + (double)(p.K / v.bk) * per_pair;
+}
+
+int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
+{
+    // Candidates from large tiles to small, of two kernels for one tile the ping-pong form first;
+    // a later candidate replaces an earlier one only when it is estimated 3 % faster.
     std::vector<int> order;
     for (int i = 0; i < miw::tiled_variant_count(); i++) order.push_back(i);
     std::stable_sort(order.begin(), order.end(), [](int a, int b) {
@@ -201,16 +214,12 @@ int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc,
         if (va.bm * va.bn != vb.bm * vb.bn) return va.bm * va.bn > vb.bm * vb.bn;
         return va.kind > vb.kind;
     });
+    int best = -1;
+    double best_us = 0.0;
     for (int i : order) {
         if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk)) continue;
-        const miw::tiled_variant &v = miw::tiled_variant_at(i);
-        const long wgs = (I / v.bm) * (J / v.bn) * p.batch;
-        // A deep LDS ring on a small tile pays when one workgroup per CU runs a long K loop;
-        // with more workgroups than CUs the shallow ring lets two of them share a CU.
-        const bool deep_small = v.stages > 2 && v.bm * v.bn <= 128 * 128 && v.bm >= 128;
-        if (deep_small && (wgs > cus || p.K / v.bk < 2 * v.stages)) continue;
-        if (wgs >= cus) return i + 1;
-        if (wgs > best_wgs) { best = i; best_wgs = wgs; }
+        const double us = estimate_us(i, p, c_type, d_type);
+        if (best < 0 || us < 0.97 * best_us) { best = i; best_us = us; }
     }
     if (best >= 0) return best + 1;
     return miw::tiled_variant_count() + 1;  // fragment-op kernel
@@ -668,38 +677,40 @@ int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void
     if (d->variant != 0) return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: the variant is chosen per slice; desc.variant must be 0");
     if (splits < 0 || splits > 256) return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: splits must be 0 (choose) or 1..256, got %d", splits);
     const int nt = miw::tiled_variant_count();
-    const int cus = g_cu_count > 0 ? g_cu_count : 256;
     static char dummy alignas(16);
-    auto try_splits = [&](int s, int *variant, long *wgs) {
+    // Variant and estimated duration of s slices (s = 1: the plain launch); false when no tiled kernel fits.
+    auto try_splits = [&](int s, int *variant, double *us) {
         if (p.K % (64l * s)) return false;
+        if (s == 1) {
+            const int v = pick_variant(p, d->c_type, d->d_type, false, 0);
+            if (v == nt + 1) return false;
+            *variant = v;
+            *us = estimate_us(v - 1, p, d->c_type, d->d_type);
+            return true;
+        }
         const miw::gemm_params q = splitk_slices(p, s, &dummy);
         const int v = pick_variant(q, MIW_F32, MIW_F32, false, 0);
         if (v == nt + 1) return false;
-        const miw::tiled_variant &tv = miw::tiled_variant_at(v - 1);
-        const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
         *variant = v;
-        *wgs = (I / tv.bm) * (J / tv.bn) * s;
+        // second kernel: launch, a quarter of a microsecond per slice (each thread adds its slices
+        // in order), and the slices, C and D at the same pace as above
+        const double mn = (double)p.M * (double)p.N;
+        *us = estimate_us(v - 1, q, MIW_F32, MIW_F32) + 6.0 + 0.25 * s +
+              mn * (4.0 * s + (double)dtype_size(d->d_type) + (p.use_c ? (double)dtype_size(d->c_type) : 0.0)) / 5.5e6;
         return true;
     };
     int variant = 0;
-    long wgs = 0;
+    double us = 0.0;
     if (splits == 0) {
-        // Fewest slices that give every CU a workgroup: first with tiles of at least 128 x 128 and up
-        // to 16 slices of four LDS slots' worth of K or more (large tiles move less data per flop
-        // than a small tile saves in workspace traffic), else with any tile and up to 64 slices.
-        int best = 0;
-        for (int pass = 0; pass < 2 && (best == 0 || wgs < cus); pass++)
-            for (int s = 1; s <= (pass ? 64 : 16) && p.K / s >= (pass ? 128 : 256); s++) {
-                int v;
-                long w;
-                if (!try_splits(s, &v, &w)) continue;
-                const miw::tiled_variant &tv = miw::tiled_variant_at(v - 1);
-                if (pass == 0 && (w < cus || tv.bm * tv.bn < 128 * 128)) continue;
-                best = s; variant = v; wgs = w;
-                if (w >= cus) break;
-            }
-        splits = best;
-    } else if (!try_splits(splits, &variant, &wgs)) {
+        // The slice count with the shortest estimated duration, among 1 (no second pass) and the
+        // counts up to 64 that leave every slice two LDS slots' worth of K or more.
+        double best_us = 0.0;
+        for (int s = 1; s <= 64 && (s == 1 || p.K / s >= 128); s++) {
+            int v;
+            if (!try_splits(s, &v, &us)) continue;
+            if (splits == 0 || us < 0.97 * best_us) { splits = s; variant = v; best_us = us; }
+        }
+    } else if (!try_splits(splits, &variant, &us)) {
         splits = 0;
     }
     if (splits == 0)
@@ -709,13 +720,20 @@ int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void
     out->full = p;
     out->splits = splits;
     out->variant = variant;
-    out->bytes = (size_t)splits * (size_t)p.M * (size_t)p.N * sizeof(float);
+    // one slice is the plain launch: no workspace, no second kernel
+    out->bytes = splits == 1 ? 0 : (size_t)splits * (size_t)p.M * (size_t)p.N * sizeof(float);
     out->slice = splitk_slices(p, splits, nullptr);
     return 0;
 }
 
 int run_splitk(const miw_gemm_desc *d, splitk_plan &plan, void *ws, hipStream_t s)
 {
+    if (plan.splits == 1) {
+        if (!tiled_fits(plan.variant - 1, plan.full, d->c_type, d->d_type, false, 0))
+            return fail(MIW_ERR_MISALIGNED, "gemm_splitk: operands must be 16-byte aligned");
+        HIP_TRY(miw::launch_gemm_tiled(plan.variant - 1, plan.full, d->c_type, d->d_type, false, s));
+        return 0;
+    }
     plan.slice.D = ws;
     // the slices are checked against the real operand pointers (plan_splitk assumed aligned ones)
     if (!tiled_fits(plan.variant - 1, plan.slice, MIW_F32, MIW_F32, false, 0))
@@ -745,7 +763,7 @@ int miw_gemm_splitk(const miw_gemm_desc *desc, const void *A, const void *B, con
 {
     splitk_plan plan;
     if (int rc = plan_splitk(desc, A, B, C, D, splits, &plan)) return rc;
-    if (!workspace) return fail(MIW_ERR_NULL_POINTER, "gemm_splitk: null workspace");
+    if (!workspace && plan.bytes) return fail(MIW_ERR_NULL_POINTER, "gemm_splitk: null workspace");
     if (workspace_bytes < plan.bytes)
         return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: workspace of %zu bytes, %d slices need %zu", workspace_bytes,
                     plan.splits, plan.bytes);

@@ -12,19 +12,20 @@ namespace miw {
 // --------------------------------------------------------------- variants --
 
 static const tiled_variant g_variants[] = {
-    // name                    bm   bn  bk     wm wn slots lds, kind (32-k ping-pong: ring depth of a K-major operand, largest ring)
-    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2, 0},
-    {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2, 0},
-    {"tile256x128_w4x2", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 0},
-    {"tile128x256_w2x4", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 0},
-    {"tile128x128_w2x4_s4", 128, 128, KGRAN, 2, 4, 4, 4 * (128 + 128) * KGRAN * 2, 0},
-    {"tile128x128_w2x2_s4", 128, 128, KGRAN, 2, 2, 4, 4 * (128 + 128) * KGRAN * 2, 0},
-    {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2, 0},
-    {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, 4, 4 * (64 + 64) * KGRAN * 2, 0},
-    {"tile256x256_pingpong", 256, 256, KGRAN, 2, 4, 3, 160 * 1024, 1},
-    {"tile256x128_pingpong", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 2},
-    {"tile128x256_pingpong", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 2},
-    {"tile128x128_pingpong", 128, 128, KGRAN, 4, 2, 4, 4 * (128 + 128) * KGRAN * 2, 2},
+    // name                    bm   bn  bk     wm wn slots lds, kind (32-k ping-pong: ring depth of a K-major operand, largest ring),
+    //                                                          workgroups per CU, us per 64 k alone, us per 64 k in a queue
+    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2, 0, 1, 1.37f, 1.37f},
+    {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2, 0, 1, 1.55f, 1.55f},
+    {"tile256x128_w4x2", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 0, 1, 0.80f, 0.80f},
+    {"tile128x256_w2x4", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 0, 1, 0.80f, 0.80f},
+    {"tile128x128_w2x4_s4", 128, 128, KGRAN, 2, 4, 4, 4 * (128 + 128) * KGRAN * 2, 0, 1, 0.50f, 0.50f},
+    {"tile128x128_w2x2_s4", 128, 128, KGRAN, 2, 2, 4, 4 * (128 + 128) * KGRAN * 2, 0, 1, 0.50f, 0.50f},
+    {"tile128x128_w2x2", 128, 128, KGRAN, 2, 2, 2, 2 * (128 + 128) * KGRAN * 2, 0, 2, 0.63f, 0.455f},
+    {"tile64x64_w2x2", 64, 64, KGRAN, 2, 2, 4, 4 * (64 + 64) * KGRAN * 2, 0, 2, 0.22f, 0.19f},
+    {"tile256x256_pingpong", 256, 256, KGRAN, 2, 4, 3, 160 * 1024, 1, 1, 1.30f, 1.30f},
+    {"tile256x128_pingpong", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 2, 1, 0.785f, 0.785f},
+    {"tile128x256_pingpong", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 2, 1, 0.785f, 0.785f},
+    {"tile128x128_pingpong", 128, 128, KGRAN, 4, 2, 4, 4 * (128 + 128) * KGRAN * 2, 2, 1, 0.50f, 0.50f},
 };
 
 int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }

@@ -50,6 +50,12 @@ struct tiled_variant {
     const char *name;
     int bm, bn, bk, wm, wn, stages, lds_bytes;
     int kind;  // KIND_*
+    // What the variant picker prices a launch with (measured on MI355X, U[-1,1] operands, all CUs
+    // busy, i.e. under the power cap): workgroups that fit on one CU together, microseconds per
+    // 64 k-values for a workgroup that has its CU to itself, and microseconds per 64 k-values and
+    // workgroup when a CU works through a queue of them.
+    int occupancy;
+    float us_pair_alone, us_pair_queued;
 };
 int tiled_variant_count();
 const tiled_variant &tiled_variant_at(int i);

@@ -62,7 +62,7 @@ def gemm_splitk(A, B, C, D, desc, splits=0, workspace=None, stream=None):
     `workspace` (a DeviceArray; allocated here when None) and are added in order by a second kernel."""
     n, nbytes = splitk_workspace(desc, splits)
     if workspace is None:
-        workspace = DeviceArray.undef(np.float32, nbytes // 4)
+        workspace = DeviceArray.undef(np.float32, max(nbytes // 4, 4))
     _lib.check(_lib.load().miw_gemm_splitk(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), n, _ptr(workspace),
                                            workspace.nbytes, _stream(stream)))
     return workspace

@@ -206,7 +206,9 @@ int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
 /* *supported = 1 when `variant` (1..count) can run this descriptor (tile divisibility, leading
    dimensions, operand layouts, accumulate type; pointers are assumed 16-byte aligned), else 0. */
 int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *supported);
-/* Variant miw_gemm would pick for this descriptor. */
+/* Variant miw_gemm would pick for this descriptor: the one with the shortest estimated duration
+   (rounds of workgroups over the CUs, C and D traffic, and the K loop at each kernel's measured
+   pace per 64 k-values) among those that can run it. */
 int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant);
 /* acc_chunk miw_gemm would use for this descriptor (fp16 accumulate only). */
 int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk);
@@ -218,8 +220,10 @@ int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk);
    adds the slices in order: D = alpha * sum_s A_s*B_s + beta*C.  The result does not depend on
    timing; it differs from miw_gemm's by the rounding of one Float32 sum per slice.  Float32
    accumulation, batch 1, desc.variant 0, M and N divisible by an LDS tile.  splits = 0 chooses
-   the fewest slices that give every CU a workgroup.  miw_gemm_splitk_workspace reports the slice
-   count and the bytes miw_gemm_splitk will ask for. */
+   the slice count with the shortest estimated duration (both kernels and the workspace traffic
+   counted).  One slice, asked for or chosen, is the plain launch of miw_gemm: no workspace
+   (0 bytes, `workspace` may be null) and no second kernel.  miw_gemm_splitk_workspace reports
+   the slice count and the bytes miw_gemm_splitk will ask for. */
 int miw_gemm_splitk_workspace(const miw_gemm_desc *desc, int splits, int *splits_out, size_t *bytes);
 int miw_gemm_splitk(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
                     void *workspace, size_t workspace_bytes, void *stream);

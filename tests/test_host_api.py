@@ -216,6 +216,21 @@ def test_variant_table_and_selection(miw):
     assert deep["block"][:2] == (128, 128) and deep["stages"] == 4            # one workgroup per CU, long K
     assert G.pick_variant(G.make_desc(48, 48, 48)) == by["fragment_ops"]
     assert G.pick_variant(G.make_desc(64, 64, 80)) == by["fragment_ops"]
+    # the choice goes by estimated duration, not by tile count alone:
+    # 3072^3 is 144 tiles of 256 x 256 (one round on 256 CUs) or 288 of 256 x 128 (two rounds)
+    assert vs[G.pick_variant(G.make_desc(3072, 3072, 3072)) - 1]["name"] == "tile256x256_pingpong"
+    # 1536^3: 144 tiles of 128 x 128 with a K loop half as long per flop as 576 tiles of 64 x 64
+    assert vs[G.pick_variant(G.make_desc(1536, 1536, 1536)) - 1]["block"][:2] == (128, 128)
+    # 8192 x 1024 x 4096 (A row-major): 128 tiles of 256 x 256 would leave half the CUs idle
+    c4 = G.make_desc(8192, 1024, 4096, a_layout=W.RowMajor, b_layout=W.ColMajor)
+    assert vs[G.pick_variant(c4) - 1]["name"] == "tile256x128_pingpong"
+    # few tiles and a short K: small tiles spread over more CUs
+    assert vs[G.pick_variant(G.make_desc(512, 512, 512)) - 1]["block"][:2] == (64, 64)
+    # split-K slice counts by the same estimate: none where the tiles fill the chip or K is short, several for a long K
+    assert G.splitk_workspace(G.make_desc(4096, 4096, 4096)) == (1, 0)
+    assert G.splitk_workspace(G.make_desc(256, 256, 2048)) == (1, 0)
+    n, nbytes = G.splitk_workspace(G.make_desc(256, 256, 65536))
+    assert 4 <= n <= 64 and nbytes == n * 256 * 256 * 4
     d = G.make_desc(2048, 2048, 2048, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
     assert G.acc_chunk(d) == 64
     d = G.make_desc(48, 48, 48, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
