@@ -75,6 +75,12 @@ class GemmDesc(ctypes.Structure):
     ]
 
 
+class GemmPart(ctypes.Structure):
+    _fields_ = [("variant", ctypes.c_int), ("reserved", ctypes.c_int),
+                ("m0", ctypes.c_int64), ("n0", ctypes.c_int64), ("k0", ctypes.c_int64),
+                ("m", ctypes.c_int64), ("n", ctypes.c_int64), ("k", ctypes.c_int64)]
+
+
 class GemmVariantInfo(ctypes.Structure):
     _fields_ = [
         ("name", ctypes.c_char * 64),
@@ -133,6 +139,7 @@ SIGNATURES = {
     "miw_build_id": (ctypes.c_char_p, []),
     "miw_gemm_variant_supports": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(_i)]),
     "miw_gemm_pick_variant": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
+    "miw_gemm_plan": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(GemmPart), _i, ctypes.POINTER(_i)]),
     "miw_gemm_acc_chunk": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
     "miw_gemm_splitk_workspace": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
     "miw_gemm_splitk": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),

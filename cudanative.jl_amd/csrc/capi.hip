@@ -149,12 +149,15 @@ int resolve_gemm(const miw_gemm_desc *d, const void *A, const void *B, const voi
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // Can tiled variant i (0-based) run this problem?
-bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
+// Where the tile does not divide M or N the edge tiles overlap their neighbours (both compute the
+// overlap), which C and D sharing memory (in_place) forbids.
+bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk, bool in_place)
 {
     const miw::tiled_variant &v = miw::tiled_variant_at(i);
     // In canonical terms bm tiles the contiguous dimension of D.
     const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
-    if (I % v.bm || J % v.bn || p.K % v.bk) return false;
+    if (I < v.bm || J < v.bn || p.K % v.bk) return false;
+    if ((I % v.bm || J % v.bn) && in_place) return false;
     if (!miw::tiled_supports_layout(i, p) || !miw::tiled_grid_fits(i, p)) return false;
     if (!aligned16(p.A) || !aligned16(p.B) || !aligned16(p.D) || (p.use_c && !aligned16(p.C))) return false;
     if (p.lda % 8 || p.ldb % 8 || p.sa % 8 || p.sb % 8) return false;
@@ -195,7 +198,7 @@ double estimate_us(int i, const miw::gemm_params &p, int c_type, int d_type)
     const miw::tiled_variant &v = miw::tiled_variant_at(i);
     const int cus = g_cu_count > 0 ? g_cu_count : 256;
     const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
-    const long tiles = (I / v.bm) * (J / v.bn) * p.batch;
+    const long tiles = ((I + v.bm - 1) / v.bm) * ((J + v.bn - 1) / v.bn) * p.batch;  // edge tiles overlap their neighbours
     const long per_cu = (tiles + cus - 1) / cus;
     const long rounds = (per_cu + v.occupancy - 1) / v.occupancy;
     const double per_pair = std::max((double)v.us_pair_alone, (double)per_cu * v.us_pair_queued);
@@ -203,21 +206,30 @@ double estimate_us(int i, const miw::gemm_params &p, int c_type, int d_type)
     return 4.5 * (double)rounds + cd_bytes / 5.5e6 + (double)(p.K / v.bk) * per_pair;
 }
 
-int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk)
+// Tiled variants from large tiles to small, of two kernels for one tile the ping-pong form first.
+const std::vector<int> &variant_order()
 {
-    // Candidates from large tiles to small, of two kernels for one tile the ping-pong form first;
-    // a later candidate replaces an earlier one only when it is estimated 3 % faster.
-    std::vector<int> order;
-    for (int i = 0; i < miw::tiled_variant_count(); i++) order.push_back(i);
-    std::stable_sort(order.begin(), order.end(), [](int a, int b) {
-        const miw::tiled_variant &va = miw::tiled_variant_at(a), &vb = miw::tiled_variant_at(b);
-        if (va.bm * va.bn != vb.bm * vb.bn) return va.bm * va.bn > vb.bm * vb.bn;
-        return va.kind > vb.kind;
-    });
+    static const std::vector<int> order = [] {
+        std::vector<int> o;
+        for (int i = 0; i < miw::tiled_variant_count(); i++) o.push_back(i);
+        std::stable_sort(o.begin(), o.end(), [](int a, int b) {
+            const miw::tiled_variant &va = miw::tiled_variant_at(a), &vb = miw::tiled_variant_at(b);
+            if (va.bm * va.bn != vb.bm * vb.bn) return va.bm * va.bn > vb.bm * vb.bn;
+            return va.kind > vb.kind;
+        });
+        return o;
+    }();
+    return order;
+}
+
+int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc, int acc_chunk, bool in_place)
+{
+    // Candidates in the order of variant_order(); a later candidate replaces an earlier one only when it is estimated 3 % faster.
+    const std::vector<int> &order = variant_order();
     int best = -1;
     double best_us = 0.0;
     for (int i : order) {
-        if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk)) continue;
+        if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk, in_place)) continue;
         const double us = estimate_us(i, p, c_type, d_type);
         if (best < 0 || us < 0.97 * best_us) { best = i; best_us = us; }
     }
@@ -226,12 +238,12 @@ int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc,
 }
 
 // Resolve the variant (0 = pick) and check that it can run this problem; touches no device.
-int check_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, int *variant_out)
+int check_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, bool in_place, int *variant_out)
 {
     const int nt = miw::tiled_variant_count();
     int variant = d->variant;
     if (variant < 0 || variant > nt + 1) return fail(MIW_ERR_INVALID_VALUE, "gemm: unknown variant %d", variant);
-    if (variant == 0) variant = pick_variant(p, d->c_type, d->d_type, f16acc, d->acc_chunk);
+    if (variant == 0) variant = pick_variant(p, d->c_type, d->d_type, f16acc, d->acc_chunk, in_place);
     if (variant == nt + 1) {
         if (f16acc && d->acc_chunk != 0 && d->acc_chunk != 16)
             return fail(MIW_ERR_UNSUPPORTED, "gemm: the fragment-op kernel rounds every 16 k-values (acc_chunk %d asked)",
@@ -239,9 +251,10 @@ int check_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, i
         if ((p.M / 16) * (p.N / 16) / 4 >= (1l << 31))
             return fail(MIW_ERR_UNSUPPORTED, "gemm: %lld x %lld tiles of 16 x 16 do not fit the launch grid",
                         (long long)(p.M / 16), (long long)(p.N / 16));
-    } else if (!tiled_fits(variant - 1, p, d->c_type, d->d_type, f16acc, d->acc_chunk)) {
+    } else if (!tiled_fits(variant - 1, p, d->c_type, d->d_type, f16acc, d->acc_chunk, in_place)) {
         return fail(MIW_ERR_UNSUPPORTED,
-                    "gemm: variant %d (%s) needs tile-divisible sizes, 16-byte aligned operands and leading "
+                    "gemm: variant %d (%s) needs M and N of at least one tile (whole tiles when C and D share memory), "
+                    "K divisible by 64, 16-byte aligned operands and leading "
                     "dimensions, a tile count that fits the launch grid, and (ping-pong kernels) at most one operand "
                     "with k contiguous%s",
                     variant, miw::tiled_variant_at(variant - 1).name,
@@ -251,10 +264,174 @@ int check_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, i
     return 0;
 }
 
-int launch_gemm(int variant, const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, hipStream_t s)
+int launch_gemm(int variant, const miw::gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s)
 {
-    if (variant == miw::tiled_variant_count() + 1) HIP_TRY(miw::launch_gemm_fragops(p, d->c_type, d->d_type, f16acc, s));
-    else HIP_TRY(miw::launch_gemm_tiled(variant - 1, p, d->c_type, d->d_type, f16acc, s));
+    if (variant == miw::tiled_variant_count() + 1) HIP_TRY(miw::launch_gemm_fragops(p, c_type, d_type, f16acc, s));
+    else HIP_TRY(miw::launch_gemm_tiled(variant - 1, p, c_type, d_type, f16acc, s));
+    return 0;
+}
+
+// ---- ragged problems ----
+// The tiled kernels take any M and N of at least one tile: where the tile does not divide an
+// extent the last tile is shifted back to end at the edge and overlaps its neighbour (unless C
+// and D share memory: then only whole tiles).  Beyond that a problem may be cut into parts, each
+// a GEMM of its own on a block of D (same leading dimensions and batch strides, offset
+// pointers), launched one after the other on the caller's stream:
+//   * K = 64 q + r (Float32 D): the first 64 q k-values by the tiled kernels, the last r by the
+//     fragment-op kernel with D as its C operand (one more Float32 rounding per element);
+//   * a body of whole large tiles plus a bottom strip and a right strip, each planned again
+//     (4160 rows: sixteen rows of 256 x 256 tiles and a strip of 64 x 64 tiles instead of
+//     seventeen rows of large tiles, i.e. two rounds over the CUs).
+// A cut is made only where the estimate says it pays.
+struct gemm_part {
+    int variant;  // 1-based; tiled_variant_count() + 1: the fragment-op kernel
+    int c_type;
+    miw::gemm_params p;
+    long m0, n0, k0;  // where the part sits in the caller's problem
+};
+
+// The fragment-op kernel: every wavefront walks K alone, 16 k-values per step, straight from global memory.
+double estimate_fragops_us(const miw::gemm_params &p, int c_type, int d_type)
+{
+    const double mn = (double)p.M * (double)p.N * (double)p.batch;
+    const double walk = 0.45 * (double)(p.K / 16);
+    const double flops = 2.0 * mn * (double)p.K / 45e6;
+    const double bytes = mn * (double)(dtype_size(d_type) + (p.use_c ? dtype_size(c_type) : 0)) / 2.0e6;
+    return 5.0 + std::max(walk, std::max(flops, bytes));
+}
+
+miw::gemm_params sub_block(const miw::gemm_params &p, int c_type, int d_type, long m0, long m, long n0, long n)
+{
+    miw::gemm_params q = p;
+    q.A = p.A + m0 * (p.a_row ? p.lda : 1);
+    q.B = p.B + n0 * (p.b_row ? 1 : p.ldb);
+    if (p.C) q.C = (const char *)p.C + (long)dtype_size(c_type) * (p.c_row ? m0 * p.ldc + n0 : n0 * p.ldc + m0);
+    q.D = (char *)p.D + (long)dtype_size(d_type) * (p.d_row ? m0 * p.ldd + n0 : n0 * p.ldd + m0);
+    q.M = m;
+    q.N = n;
+    return q;
+}
+
+struct gemm_planner {
+    int d_type;
+    bool in_place;  // C and D share memory
+    int nt = miw::tiled_variant_count();
+
+    double single(const miw::gemm_params &p, int c_type, long m0, long n0, long k0, std::vector<gemm_part> *out) const
+    {
+        const int v = pick_variant(p, c_type, d_type, false, 0, in_place);
+        if (out) out->push_back(gemm_part{v, c_type, p, m0, n0, k0});
+        return v == nt + 1 ? estimate_fragops_us(p, c_type, d_type) : estimate_us(v - 1, p, c_type, d_type);
+    }
+
+    // Appends the parts of p to *out (when given) and returns the estimated duration.
+    double plan(const miw::gemm_params &p, int c_type, long m0, long n0, long k0, int depth, std::vector<gemm_part> *out) const
+    {
+        std::vector<gemm_part> best;
+        double best_us = single(p, c_type, m0, n0, k0, &best);
+        auto offer = [&](std::vector<gemm_part> &cand, double us) {
+            if (us < 0.97 * best_us) { best_us = us; best.swap(cand); }
+        };
+        if (depth < 4) {
+            const long k64 = p.K / 64 * 64;
+            if (k64 != p.K && k64 > 0 && d_type == MIW_F32) {
+                miw::gemm_params body = p, tail = p;
+                body.K = k64;
+                tail.K = p.K - k64;
+                tail.A = p.A + k64 * (p.a_row ? 1 : p.lda);
+                tail.B = p.B + k64 * (p.b_row ? p.ldb : 1);
+                tail.C = p.D; tail.use_c = 1; tail.beta = 1.0f;
+                tail.c_row = p.d_row; tail.ldc = p.ldd; tail.sc = p.sd;
+                std::vector<gemm_part> cand;
+                double us = plan(body, c_type, m0, n0, k0, depth + 1, &cand);
+                us += single(tail, d_type, m0, n0, k0 + k64, &cand);
+                offer(cand, us);
+            } else if (k64 == p.K) {
+                // whole large tiles, then what they leave at the bottom and on the right; a strip
+                // is widened backwards to 64 rows (columns), over the body, where that is allowed
+                for (int i : variant_order()) {
+                    const miw::tiled_variant &v = miw::tiled_variant_at(i);
+                    const long tm = p.d_row ? v.bn : v.bm, tn = p.d_row ? v.bm : v.bn;
+                    const long mb = p.M / tm * tm, nb = p.N / tn * tn;
+                    if (mb == 0 || nb == 0 || (mb == p.M && nb == p.N)) continue;
+                    const miw::gemm_params body = sub_block(p, c_type, d_type, 0, mb, 0, nb);
+                    if (!tiled_fits(i, body, c_type, d_type, false, 0, in_place)) continue;
+                    std::vector<gemm_part> cand;
+                    cand.push_back(gemm_part{i + 1, c_type, body, m0, n0, k0});
+                    double us = estimate_us(i, body, c_type, d_type);
+                    if (us >= best_us) continue;
+                    const long sm = in_place || p.M < 64 ? mb : std::min(mb, p.M - 64);
+                    const long sn = in_place || p.N < 64 ? nb : std::min(nb, p.N - 64);
+                    if (mb != p.M)
+                        us += plan(sub_block(p, c_type, d_type, sm, p.M - sm, 0, p.N), c_type, m0 + sm, n0, k0, depth + 1, &cand);
+                    if (nb != p.N)
+                        us += plan(sub_block(p, c_type, d_type, 0, mb, sn, p.N - sn), c_type, m0, n0 + sn, k0, depth + 1, &cand);
+                    offer(cand, us);
+                }
+            }
+        }
+        if (out) out->insert(out->end(), best.begin(), best.end());
+        return best_us;
+    }
+};
+
+bool ranges_overlap(const void *a, size_t na, const void *b, size_t nb)
+{
+    const uintptr_t x = (uintptr_t)a, y = (uintptr_t)b;
+    return x < y + nb && y < x + na;
+}
+
+// The launches of one miw_gemm call, validated.  A forced variant and fp16 accumulation (whose
+// rounding points must not depend on where a cut falls) run as one launch.
+int plan_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, bool in_place, std::vector<gemm_part> *parts)
+{
+    // The host thread's last plan is kept: a loop over one problem and one set of buffers plans once.
+    struct cached_plan {
+        miw_gemm_desc desc;
+        const void *A, *B, *C;
+        void *D;
+        bool in_place, valid = false;
+        std::vector<gemm_part> parts;
+    };
+    static thread_local cached_plan last;
+    if (last.valid && memcmp(&last.desc, d, sizeof *d) == 0 && last.A == p.A && last.B == p.B && last.C == p.C && last.D == p.D &&
+        last.in_place == in_place) {
+        *parts = last.parts;
+        return 0;
+    }
+    parts->clear();
+    if (d->variant != 0 || f16acc) {
+        int variant = 0;
+        if (int rc = check_gemm(d, p, f16acc, in_place, &variant)) return rc;
+        parts->push_back(gemm_part{variant, d->c_type, p, 0, 0, 0});
+    } else {
+        gemm_planner pl{d->d_type, in_place};
+        pl.plan(p, d->c_type, 0, 0, 0, 0, parts);
+        for (const gemm_part &part : *parts)
+            if (part.variant == pl.nt + 1 && (part.p.M / 16) * (part.p.N / 16) / 4 >= (1l << 31))
+                return fail(MIW_ERR_UNSUPPORTED, "gemm: %lld x %lld tiles of 16 x 16 do not fit the launch grid",
+                            (long long)(part.p.M / 16), (long long)(part.p.N / 16));
+    }
+    last.desc = *d;
+    last.A = p.A; last.B = p.B; last.C = p.C; last.D = p.D;
+    last.in_place = in_place;
+    last.parts = *parts;
+    last.valid = true;
+    return 0;
+}
+
+bool c_shares_d(const miw_gemm_desc *d, const miw::gemm_params &p)
+{
+    if (!p.use_c) return false;
+    const size_t nc = (size_t)((p.batch - 1) * p.sc + p.ldc * (p.c_row ? p.M : p.N)) * dtype_size(d->c_type);
+    const size_t nd = (size_t)((p.batch - 1) * p.sd + p.ldd * (p.d_row ? p.M : p.N)) * dtype_size(d->d_type);
+    return ranges_overlap(p.C, nc, p.D, nd);
+}
+
+int launch_parts(const miw_gemm_desc *d, const std::vector<gemm_part> &parts, bool f16acc, hipStream_t s)
+{
+    for (const gemm_part &part : parts)
+        if (int rc = launch_gemm(part.variant, part.p, part.c_type, d->d_type, f16acc, s)) return rc;
     return 0;
 }
 
@@ -573,7 +750,7 @@ int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *suppo
     static char dummy alignas(16);
     if (int rc = resolve_gemm(desc, &dummy, &dummy, &dummy, &dummy, &p, &f16acc)) return rc;
     if (variant == nt + 1) *supported = !(f16acc && desc->acc_chunk != 0 && desc->acc_chunk != 16);
-    else *supported = tiled_fits(variant - 1, p, desc->c_type, desc->d_type, f16acc, desc->acc_chunk) ? 1 : 0;
+    else *supported = tiled_fits(variant - 1, p, desc->c_type, desc->d_type, f16acc, desc->acc_chunk, false) ? 1 : 0;
     return 0;
 }
 
@@ -585,7 +762,29 @@ int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant)
     // Alignment of real pointers cannot be known here: assume aligned operands.
     static char dummy alignas(16);
     if (int rc = resolve_gemm(desc, &dummy, &dummy, &dummy, &dummy, &p, &f16acc)) return rc;
-    *variant = pick_variant(p, desc->c_type, desc->d_type, f16acc, desc->acc_chunk);
+    *variant = pick_variant(p, desc->c_type, desc->d_type, f16acc, desc->acc_chunk, false);
+    return 0;
+}
+
+int miw_gemm_plan(const miw_gemm_desc *desc, int in_place, miw_gemm_part *out, int capacity, int *count)
+{
+    if (!count || (capacity > 0 && !out)) return fail(MIW_ERR_NULL_POINTER, "gemm_plan: null output");
+    miw::gemm_params p;
+    bool f16acc;
+    // Alignment of real pointers cannot be known here: assume 16-byte aligned operands far apart.
+    char *const base = (char *)(uintptr_t)0x100000000ull;
+    if (int rc = resolve_gemm(desc, base, base + (1ull << 40), base + (2ull << 40), base + (in_place ? 2ull << 40 : 3ull << 40), &p, &f16acc))
+        return rc;
+    std::vector<gemm_part> parts;
+    if (int rc = plan_gemm(desc, p, f16acc, in_place != 0, &parts)) return rc;
+    *count = (int)parts.size();
+    for (int i = 0; i < (int)parts.size() && i < capacity; i++) {
+        const gemm_part &g = parts[(size_t)i];
+        out[i].variant = g.variant;
+        out[i].reserved = 0;
+        out[i].m0 = g.m0; out[i].n0 = g.n0; out[i].k0 = g.k0;
+        out[i].m = g.p.M; out[i].n = g.p.N; out[i].k = g.p.K;
+    }
     return 0;
 }
 
@@ -603,11 +802,11 @@ int miw_gemm(const miw_gemm_desc *desc, const void *A, const void *B, const void
 {
     miw::gemm_params p;
     bool f16acc;
-    int variant = 0;
     if (int rc = resolve_gemm(desc, A, B, C, D, &p, &f16acc)) return rc;
-    if (int rc = check_gemm(desc, p, f16acc, &variant)) return rc;
+    std::vector<gemm_part> parts;
+    if (int rc = plan_gemm(desc, p, f16acc, c_shares_d(desc, p), &parts)) return rc;
     REQUIRE_INIT("gemm");
-    return launch_gemm(variant, desc, p, f16acc, as_stream(stream));
+    return launch_parts(desc, parts, f16acc, as_stream(stream));
 }
 
 // ---- split-K ----
@@ -677,19 +876,20 @@ int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void
     if (d->variant != 0) return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: the variant is chosen per slice; desc.variant must be 0");
     if (splits < 0 || splits > 256) return fail(MIW_ERR_INVALID_VALUE, "gemm_splitk: splits must be 0 (choose) or 1..256, got %d", splits);
     const int nt = miw::tiled_variant_count();
+    const bool in_place = c_shares_d(d, p);
     static char dummy alignas(16);
     // Variant and estimated duration of s slices (s = 1: the plain launch); false when no tiled kernel fits.
     auto try_splits = [&](int s, int *variant, double *us) {
         if (p.K % (64l * s)) return false;
         if (s == 1) {
-            const int v = pick_variant(p, d->c_type, d->d_type, false, 0);
+            const int v = pick_variant(p, d->c_type, d->d_type, false, 0, in_place);
             if (v == nt + 1) return false;
             *variant = v;
             *us = estimate_us(v - 1, p, d->c_type, d->d_type);
             return true;
         }
         const miw::gemm_params q = splitk_slices(p, s, &dummy);
-        const int v = pick_variant(q, MIW_F32, MIW_F32, false, 0);
+        const int v = pick_variant(q, MIW_F32, MIW_F32, false, 0, false);
         if (v == nt + 1) return false;
         *variant = v;
         // second kernel: launch, a quarter of a microsecond per slice (each thread adds its slices
@@ -729,14 +929,14 @@ int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void
 int run_splitk(const miw_gemm_desc *d, splitk_plan &plan, void *ws, hipStream_t s)
 {
     if (plan.splits == 1) {
-        if (!tiled_fits(plan.variant - 1, plan.full, d->c_type, d->d_type, false, 0))
+        if (!tiled_fits(plan.variant - 1, plan.full, d->c_type, d->d_type, false, 0, c_shares_d(d, plan.full)))
             return fail(MIW_ERR_MISALIGNED, "gemm_splitk: operands must be 16-byte aligned");
         HIP_TRY(miw::launch_gemm_tiled(plan.variant - 1, plan.full, d->c_type, d->d_type, false, s));
         return 0;
     }
     plan.slice.D = ws;
     // the slices are checked against the real operand pointers (plan_splitk assumed aligned ones)
-    if (!tiled_fits(plan.variant - 1, plan.slice, MIW_F32, MIW_F32, false, 0))
+    if (!tiled_fits(plan.variant - 1, plan.slice, MIW_F32, MIW_F32, false, 0, false))
         return fail(MIW_ERR_MISALIGNED, "gemm_splitk: operands and workspace must be 16-byte aligned");
     HIP_TRY(miw::launch_gemm_tiled(plan.variant - 1, plan.slice, MIW_F32, MIW_F32, false, s));
     HIP_TRY(miw::launch_splitk_reduce(plan.full, d->c_type, d->d_type, plan.splits, (const float *)ws, s));
@@ -750,9 +950,10 @@ extern "C" {
 int miw_gemm_splitk_workspace(const miw_gemm_desc *desc, int splits, int *splits_out, size_t *bytes)
 {
     if (!bytes) return fail(MIW_ERR_NULL_POINTER, "gemm_splitk_workspace: null output");
-    static char dummy alignas(16);
+    // Alignment of real pointers cannot be known here: assume 16-byte aligned operands far apart.
+    char *const base = (char *)(uintptr_t)0x100000000ull;
     splitk_plan plan;
-    if (int rc = plan_splitk(desc, &dummy, &dummy, &dummy, &dummy, splits, &plan)) return rc;
+    if (int rc = plan_splitk(desc, base, base + (1ull << 40), base + (2ull << 40), base + (3ull << 40), splits, &plan)) return rc;
     if (splits_out) *splits_out = plan.splits;
     *bytes = plan.bytes;
     return 0;
@@ -796,13 +997,13 @@ int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, cons
         return fail(MIW_ERR_INVALID_VALUE, "gemm_bench: bad warmup/iters/output (at most 100000 timed launches per call)");
     miw::gemm_params p;
     bool f16acc;
-    int variant = 0;
     if (int rc = resolve_gemm(desc, A, B, C, D, &p, &f16acc)) return rc;
-    if (int rc = check_gemm(desc, p, f16acc, &variant)) return rc;
+    std::vector<gemm_part> parts;
+    if (int rc = plan_gemm(desc, p, f16acc, c_shares_d(desc, p), &parts)) return rc;
     REQUIRE_INIT("gemm_bench");
     hipStream_t s = as_stream(stream);
     for (int i = 0; i < warmup; i++)
-        if (int rc = launch_gemm(variant, desc, p, f16acc, s)) return rc;
+        if (int rc = launch_parts(desc, parts, f16acc, s)) return rc;
     std::vector<hipEvent_t> ev((size_t)iters + 1, nullptr);
     int rc = 0;
     hipError_t he = hipSuccess;
@@ -810,7 +1011,7 @@ int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, cons
         if (he == hipSuccess) he = hipEventCreate(&e);
     if (he == hipSuccess) he = hipEventRecord(ev[0], s);
     for (int i = 0; i < iters && rc == 0 && he == hipSuccess; i++) {
-        rc = launch_gemm(variant, desc, p, f16acc, s);
+        rc = launch_parts(desc, parts, f16acc, s);
         if (rc == 0) he = hipEventRecord(ev[(size_t)i + 1], s);
     }
     if (rc == 0 && he == hipSuccess) he = hipEventSynchronize(ev[(size_t)iters]);

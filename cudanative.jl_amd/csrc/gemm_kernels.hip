@@ -78,8 +78,9 @@ bool tiled_grid_fits(int i, const gemm_params &g)
 {
     const tiled_variant &v = g_variants[i];
     const long I = g.d_row ? g.N : g.M, J = g.d_row ? g.M : g.N;
-    const long tiles = (I / v.bm) * (J / v.bn);
-    return tiles > 0 && tiles * (long)(v.wm * v.wn * 64) < (1l << 32) && tiles <= 0x7fffffffl;
+    if (I < v.bm || J < v.bn) return false;
+    const long tiles = ((I + v.bm - 1) / v.bm) * ((J + v.bn - 1) / v.bn);
+    return tiles * (long)(v.wm * v.wn * 64) < (1l << 32) && tiles <= 0x7fffffffl;
 }
 
 // Which operands have k contiguous once the problem is in canonical form (see gemm_tiled.hpp).
@@ -137,8 +138,8 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
     p.ldc = g.ldc; p.ldd = g.ldd; p.sc = g.sc; p.sd = g.sd;
     p.use_c = g.use_c;
     p.alpha = g.alpha; p.beta = g.beta;
-    p.tiles_i = p.I / v.bm;
-    p.tiles_j = p.J / v.bn;
+    p.tiles_i = (p.I + v.bm - 1) / v.bm;
+    p.tiles_j = (p.J + v.bn - 1) / v.bn;
     // Rows of tiles per raster group: about the square root of one XCD's share.
     int per_xcd = (p.tiles_i * p.tiles_j + 7) / 8, gi = 1;
     while ((gi * 2) * (gi * 2) <= per_xcd) gi *= 2;

@@ -177,7 +177,8 @@ void k_gemm_pp(tiled_params p)
         tj0 = in / gi;
     }
     const long bt = blockIdx.y;
-    const int i0 = ti0 * BI, j0 = tj0 * BJ;
+    // the last tile of a row or column is shifted back so that it ends at the edge (see tiled_params)
+    const int i0 = min(ti0 * BI, p.I - BI), j0 = min(tj0 * BJ, p.J - BJ);
 
     const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
     const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);
@@ -548,7 +549,8 @@ void k_gemm_pp64(tiled_params p)
         tj0 = in / gi;
     }
     const long bt = blockIdx.y;
-    const int i0 = ti0 * BI, j0 = tj0 * BJ;
+    // the last tile of a row or column is shifted back so that it ends at the edge (see tiled_params)
+    const int i0 = min(ti0 * BI, p.I - BI), j0 = min(tj0 * BJ, p.J - BJ);
 
     const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
     const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);

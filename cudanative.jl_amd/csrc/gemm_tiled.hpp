@@ -69,6 +69,10 @@ struct tiled_params {
     int c_trans;  // C is stored with J contiguous (its layout differs from D's)
     int use_c;
     float alpha, beta;
+    // tiles_i = ceil(I / BI), tiles_j = ceil(J / BJ).  Where the tile does not divide an extent the
+    // last tile starts at I - BI (J - BJ) and overlaps its neighbour: both workgroups compute the
+    // overlap from the same operands in the same order and store equal values.  The host allows
+    // this only when C and D do not share memory.
     int tiles_i, tiles_j, group_i;
 #ifdef MIW_PP_TS
     long long *ts;  // measurement builds: 10 counters per wavefront (see k_gemm_pp64), or null
@@ -313,7 +317,8 @@ void k_gemm_tiled(tiled_params p)
         tj0 = in / gi;
     }
     const long bt = blockIdx.y;
-    const int i0 = ti0 * BI, j0 = tj0 * BJ;
+    // the last tile of a row or column is shifted back so that it ends at the edge (see tiled_params)
+    const int i0 = min(ti0 * BI, p.I - BI), j0 = min(tj0 * BJ, p.J - BJ);
 
     const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
     const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);

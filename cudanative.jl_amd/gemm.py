@@ -112,6 +112,17 @@ def pick_variant(desc):
     return v.value
 
 
+def plan(desc, in_place=False):
+    """The launches gemm() makes for this descriptor: a list of dicts (variant id, first row, column and
+    k-value, sizes).  One entry unless the sizes are ragged and cutting the problem up is estimated faster."""
+    lib = _lib.load()
+    n = ctypes.c_int()
+    parts = (_lib.GemmPart * 64)()
+    _lib.check(lib.miw_gemm_plan(ctypes.byref(desc), int(bool(in_place)), parts, 64, ctypes.byref(n)))
+    return [{"variant": q.variant, "m0": q.m0, "n0": q.n0, "k0": q.k0, "m": q.m, "n": q.n, "k": q.k}
+            for q in parts[:min(n.value, 64)]]
+
+
 def acc_chunk(desc):
     v = ctypes.c_int()
     _lib.check(_lib.load().miw_gemm_acc_chunk(ctypes.byref(desc), ctypes.byref(v)))

@@ -617,6 +617,13 @@ struct GemmVariantInfo
     pingpong::Cint
 end
 
+struct GemmPart
+    variant::Cint
+    reserved::Cint
+    m0::Int64; n0::Int64; k0::Int64
+    m::Int64; n::Int64; k::Int64
+end
+
 function gemm_desc(M::Integer, N::Integer, K::Integer, ::Type{CT}, ::Type{DT}; alpha=1f0, beta=1f0,
                    a_layout=WMMA.ColMajor, b_layout=WMMA.ColMajor, c_layout=WMMA.ColMajor, d_layout=WMMA.ColMajor,
                    acc_type=Float32, acc_chunk=0, use_c=true, batch=1, variant=0, lda=0, ldb=0, ldc=0, ldd=0,
@@ -662,6 +669,15 @@ function pick_variant(desc::GemmDesc)
     v = Ref{Cint}(0)
     check(ccall((:miw_gemm_pick_variant, libmiwmma), Cint, (Ptr{GemmDesc}, Ptr{Cint}), Ref(desc), v))
     return Int(v[])
+end
+
+"The launches `gemm!` makes for this descriptor (one unless the sizes are ragged and cutting pays)."
+function gemm_plan(desc::GemmDesc; in_place::Bool=false)
+    parts = Vector{GemmPart}(undef, 64)
+    n = Ref{Cint}(0)
+    check(ccall((:miw_gemm_plan, libmiwmma), Cint, (Ptr{GemmDesc}, Cint, Ptr{GemmPart}, Cint, Ptr{Cint}),
+                Ref(desc), in_place ? 1 : 0, parts, length(parts), n))
+    return parts[1:min(Int(n[]), length(parts))]
 end
 
 function variant_supports(desc::GemmDesc, variant::Integer)

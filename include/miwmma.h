@@ -206,10 +206,32 @@ int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
 /* *supported = 1 when `variant` (1..count) can run this descriptor (tile divisibility, leading
    dimensions, operand layouts, accumulate type; pointers are assumed 16-byte aligned), else 0. */
 int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *supported);
-/* Variant miw_gemm would pick for this descriptor: the one with the shortest estimated duration
+/* Variant of a single launch of this descriptor (what miw_gemm runs unless miw_gemm_plan
+   cuts the problem up): the one with the shortest estimated duration
    (rounds of workgroups over the CUs, C and D traffic, and the K loop at each kernel's measured
    pace per 64 k-values) among those that can run it. */
 int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant);
+/* The launches miw_gemm makes for this descriptor.  The LDS-tiled kernels take any M and N of
+   at least one tile (multiples of 16, as everywhere): where the tile does not divide an extent
+   the last tile is shifted back so that it ends at the edge and overlaps its neighbour; both
+   workgroups compute the overlap from the same operands in the same order and store equal
+   values.  When C and D share memory (in_place != 0 here; miw_gemm looks at the pointers) that is
+   not allowed and only whole tiles are used.  Beyond that, with Float32 accumulation and
+   desc.variant 0, a problem is cut into parts, each a GEMM on a block of D with offset pointers,
+   launched in order on the caller's stream, where the estimate says that is faster:
+     k = 64 q + r (Float32 D only): the first 64 q k-values, then the last r through the
+       fragment-op kernel with D as its C operand (one more Float32 rounding per element);
+     whole large tiles, then a bottom strip and a right strip, each planned again (4160 rows:
+       sixteen rows of 256 x 256 tiles and a strip of 64 x 64 tiles rather than seventeen rows of
+       large tiles, which would take two rounds over the CUs).
+   Writes min(*count, capacity) parts; *count is the number of launches. */
+typedef struct miw_gemm_part {
+    int variant;          /* as in miw_gemm_desc.variant */
+    int reserved;
+    int64_t m0, n0, k0;   /* first row, column and k-value of the part in the caller's problem */
+    int64_t m, n, k;      /* its sizes */
+} miw_gemm_part;
+int miw_gemm_plan(const miw_gemm_desc *desc, int in_place, miw_gemm_part *parts, int capacity, int *count);
 /* acc_chunk miw_gemm would use for this descriptor (fp16 accumulate only). */
 int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk);
 

@@ -280,6 +280,117 @@ def test_ragged_sizes_fall_back_to_fragment_ops(gpu, orc):
         assert np.all(Dm[bt * gr.stride_d + 104 * 112:(bt + 1) * gr.stride_d] == -5.0)
 
 
+def _plan(gpu, orc, g, in_place=False):
+    g = g.resolved()
+    desc = gpu.GEMM.make_desc(g.M, g.N, g.K, a_layout=_W(gpu, g.a_layout), b_layout=_W(gpu, g.b_layout),
+                              c_layout=_W(gpu, g.c_layout), d_layout=_W(gpu, g.d_layout), c_type=orc.np_dtype(g.c_type),
+                              d_type=orc.np_dtype(g.d_type), alpha=g.alpha, beta=g.beta, use_c=bool(g.use_c),
+                              batch=max(g.batch, 1), lda=g.lda, ldb=g.ldb, ldc=g.ldc, ldd=g.ldd, stride_a=g.stride_a,
+                              stride_b=g.stride_b, stride_c=g.stride_c, stride_d=g.stride_d)
+    return gpu.GEMM.plan(desc, in_place)
+
+
+@pytest.mark.parametrize("al,bl,cl,dl", [(1, 1, 1, 1), (0, 1, 1, 0), (1, 0, 0, 1), (0, 0, 0, 0)])
+def test_ragged_sizes_cut_into_tiled_parts_exact_on_integers(gpu, orc, al, bl, cl, dl):
+    """Sizes that are multiples of 16 but of no LDS tile: the tiled kernels shift their edge tiles back
+    so that they end at the edge, and the last k-values beyond a multiple of 64 go through the
+    fragment-op kernel as a second launch.  On small integers every part is exact, so the result must
+    equal the oracle bit for bit whatever the cuts, and nothing outside D's extent may be written."""
+    frag = gpu.GEMM.variants()[-1]["id"]
+    for n, (M, N, K, kw) in enumerate([(1040, 1104, 1040, {}),                       # ragged in m, n and k
+                                       (592, 656, 2064, dict(alpha=-2.0, beta=0.5)),
+                                       (2064, 80, 1024, dict(d_type=orc.F16, c_type=orc.F16)),   # narrow: two windows over n
+                                       (80, 2064, 1024, dict(use_c=0)),
+                                       (1088, 1088, 1040, dict(batch=2))]):          # only k ragged, batched
+        pad = 8 * (n % 3)
+        g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl,
+                         lda=(K if al == orc.ROW else M) + pad, ldd=(N if dl == orc.ROW else M) + 2 * pad, **kw)
+        parts = _plan(gpu, orc, g)
+        assert any(q["variant"] != frag for q in parts) and (K % 64 == 0 or len(parts) >= 2), (M, N, K, parts)
+        # the parts cover D and the K extent
+        cover = np.zeros((M, N), dtype=np.int64)
+        for q in parts:
+            cover[q["m0"]:q["m0"] + q["m"], q["n0"]:q["n0"] + q["n"]] += q["k"]
+            assert q["m"] % 16 == 0 and q["n"] % 16 == 0 and q["k"] % 16 == 0
+        assert cover.min() >= K                                                       # overlaps count twice
+        A, B, C = _inputs(orc, g, 1200 + 10 * n + al + 2 * bl, ints=True)
+        D = _run(gpu, orc, g, A, B, C if g.use_c else None, prefill=7.0)
+        want = orc.gemm(g, A, B, C)
+        gr = g.resolved()
+        nb = max(gr.batch, 1)
+        for bt in range(nb):
+            lead, other = (gr.ldd, M) if dl == orc.ROW else (gr.ldd, N)
+            got = D[bt * gr.stride_d: bt * gr.stride_d + lead * other].reshape(other, lead)
+            exp = want[bt * gr.stride_d: bt * gr.stride_d + lead * other].reshape(other, lead)
+            inner = N if dl == orc.ROW else M
+            assert np.array_equal(got[:, :inner], exp[:, :inner]), (M, N, K, al, bl, cl, dl, bt)
+            assert np.all(got[:, inner:] == 7.0)
+
+
+@pytest.mark.parametrize("al,bl,dl", itertools.product((0, 1), repeat=3))
+def test_edge_tiles_shifted_back_every_variant(gpu, orc, al, bl, dl):
+    """Every tiled variant forced on extents its tile does not divide (one tile and a bit, two tiles and
+    a bit): the last tile of each row and column overlaps its neighbour.  Bit-exact on integers with
+    Float32 and Float16 accumulation; padding beyond D's extent stays untouched."""
+    for v in _variants(gpu):
+        if v["fragment_ops"]:
+            continue
+        big = max(v["block"][:2])
+        M, N, K = big + 16, 2 * big + 48, 192
+        for f16acc in (False, True):
+            if f16acc and not v["f16_accumulate"]:
+                continue
+            t = orc.F16 if f16acc else orc.F32
+            g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, c_type=t, d_type=t,
+                             ldd=(N if dl == orc.ROW else M) + 8)
+            A, B, C = _inputs(orc, g, 1400 + v["id"], ints=True)
+            D = _run(gpu, orc, g, A, B, C, variant=v["id"], acc_type=F16 if f16acc else F32, prefill=7.0)
+            if D is None:
+                continue
+            want = orc.gemm_f16acc(g, 64, A, B, C) if f16acc else orc.gemm(g, A, B, C)
+            inner, outer = (N, M) if dl == orc.ROW else (M, N)
+            got = D.reshape(outer, inner + 8)
+            assert np.array_equal(got[:, :inner], want.reshape(outer, inner + 8)[:, :inner]), (v["name"], al, bl, dl, f16acc)
+            assert np.all(got[:, inner:] == 7.0), v["name"]
+    # C and D in one buffer: overlapping tiles are refused, whole tiles still run
+    desc = gpu.GEMM.make_desc(272, 304, 192, variant=_variants(gpu)[6]["id"], beta=0.5)
+    dA, dB = gpu.DeviceArray(np.zeros(272 * 192, dtype=F16)), gpu.DeviceArray(np.zeros(192 * 304, dtype=F16))
+    dD = gpu.DeviceArray(np.zeros(272 * 304, dtype=F32))
+    with pytest.raises(gpu.MIWError) as e:
+        gpu.GEMM.gemm(dA, dB, dD, dD, desc)
+    assert e.value.code == gpu._lib.ERR_UNSUPPORTED
+
+
+def test_ragged_sizes_random_data_and_in_place(gpu, orc):
+    """Random data against float64 (the k tail adds one Float32 rounding per element), and the in-place
+    case: with C and D one buffer the windows must not overlap what an earlier part stored."""
+    frag = gpu.GEMM.variants()[-1]["id"]
+    g = orc.GemmDesc(M=1104, N=1040, K=2064, alpha=0.75, beta=-1.25)
+    assert len(_plan(gpu, orc, g)) >= 2
+    A, B, C = _inputs(orc, g, 1300)
+    assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+    # Float16 D: the k extent is not cut (a second rounding to Float16 would show)
+    g = orc.GemmDesc(M=2064, N=80, K=1024, d_type=orc.F16)
+    A, B, C = _inputs(orc, g, 1310)
+    assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C), orc.gemm_f64(g, A, B, C)) <= 6e-4
+    g = orc.GemmDesc(M=1104, N=1040, K=1040, d_type=orc.F16)
+    assert [q["variant"] for q in _plan(gpu, orc, g)] == [frag]
+    # in place: disjoint parts only
+    for M, N, K in ((2112, 2112, 1040), (2112 + 16, 2112, 1024)):
+        g = orc.GemmDesc(M=M, N=N, K=K, beta=0.5)
+        parts = _plan(gpu, orc, g, in_place=True)
+        seen = np.zeros((M, N), dtype=np.int64)
+        for q in parts:
+            if q["k0"] == 0:
+                seen[q["m0"]:q["m0"] + q["m"], q["n0"]:q["n0"] + q["n"]] += 1
+        assert seen.min() == 1 and seen.max() == 1, (M, N, K, parts)
+        A, B, C = _inputs(orc, g, 1320 + K)
+        dA, dB, dD = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(C.copy())
+        gpu.GEMM.gemm(dA, dB, dD, dD, gpu.GEMM.make_desc(M, N, K, beta=0.5))
+        gpu.synchronize()
+        assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32, (M, N, K)
+
+
 def test_tiled_with_padded_leading_dimensions_and_batch(gpu, orc):
     g = orc.GemmDesc(M=128, N=128, K=192, lda=136, ldb=200, ldc=132, ldd=144, batch=5, a_layout=orc.COL, b_layout=orc.COL)
     A, B, C = _inputs(orc, g, 41)

@@ -13,7 +13,7 @@ JL = os.path.join(ROOT, "cudanative.jl_amd", "julia", "MIWMMA.jl")
 HDR = os.path.join(ROOT, "include", "miwmma.h")
 
 STRUCTS = {"GemmDesc": "miw_gemm_desc", "MacDesc": "miw_mac_desc", "DeviceInfo": "miw_device_info",
-           "GemmVariantInfo": "miw_gemm_variant_info", "KernelAttributes": "miw_kernel_attributes"}
+           "GemmVariantInfo": "miw_gemm_variant_info", "GemmPart": "miw_gemm_part", "KernelAttributes": "miw_kernel_attributes"}
 JL_SCALAR = {"Cint": "int", "Cuint": "unsigned", "Csize_t": "size_t", "Cfloat": "float", "Cdouble": "double",
              "Int64": "int64_t", "UInt8": "char", "Cvoid": "void"}
 
