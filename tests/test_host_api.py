@@ -140,6 +140,7 @@ def test_struct_sizes_match_header(miw):
     assert ctypes.sizeof(L.MacDesc) == 13 * 4 + 4 + 4 * 8      # 13 ints/floats, pad, 4 int64
     assert ctypes.sizeof(L.GemmDesc) == 7 * 8 + 11 * 4 + 4 + 5 * 8 + 8
     assert ctypes.sizeof(L.GemmVariantInfo) == 64 + 10 * 4
+    assert ctypes.sizeof(L.GemmPart) == 2 * 4 + 6 * 8
     assert ctypes.sizeof(L.DeviceInfo) == 128 + 64 + 7 * 4 + 4 + 2 * 8 + 8
 
 
@@ -192,6 +193,61 @@ def test_abi_rejects_bad_arguments_without_touching_the_gpu(miw):
     assert lib.miw_kernel_lookup(b"no_such_kernel", ctypes.byref(k)) == L.ERR_NOT_FOUND
     assert lib.miw_launch(ctypes.c_void_p(0x1234), (ctypes.c_uint * 3)(1, 1, 1), (ctypes.c_uint * 3)(64, 1, 1), 0, None,
                           None) == L.ERR_NOT_FOUND
+
+
+def test_gemm_plan_covers_the_problem(miw):
+    """miw_gemm_plan on seeded random sizes (host logic only): every part lies inside the problem, is a
+    multiple of 16 in every extent, names a variant that supports it, and together the parts cover every
+    element of D with exactly K k-values per element outside overlaps (at least K inside); with C and D
+    in one buffer the parts that start at k = 0 are disjoint; a forced variant and fp16 accumulation plan
+    one launch."""
+    G, W = miw.GEMM, miw.WMMA
+    vs = G.variants()
+    frag = vs[-1]["id"]
+    rng = np.random.default_rng(5)
+    layouts = (W.ColMajor, W.RowMajor)
+    cut = 0
+    for case in range(300):
+        M, N = (16 * int(rng.integers(1, 300)) for _ in range(2))
+        K = 16 * int(rng.integers(1, 300)) if case % 3 else 64 * int(rng.integers(1, 80))
+        in_place = bool(case % 4 == 1)
+        dt = np.float16 if case % 5 == 2 else np.float32
+        desc = G.make_desc(M, N, K, a_layout=layouts[case & 1], b_layout=layouts[(case >> 1) & 1],
+                           d_layout=layouts[(case >> 2) & 1], c_layout=layouts[(case >> 2) & 1], d_type=dt,
+                           batch=1 + case % 3)
+        parts = G.plan(desc, in_place)
+        assert 1 <= len(parts) <= 64
+        cut += len(parts) > 1
+        cover = np.zeros((M // 16, N // 16), dtype=np.int64)
+        first = np.zeros((M // 16, N // 16), dtype=np.int64)
+        for q in parts:
+            assert min(q["m0"], q["n0"], q["k0"]) >= 0 and min(q["m"], q["n"], q["k"]) >= 16, (M, N, K, q)
+            assert all(q[x] % 16 == 0 for x in ("m0", "n0", "k0", "m", "n", "k")), (M, N, K, q)
+            assert q["m0"] + q["m"] <= M and q["n0"] + q["n"] <= N and q["k0"] + q["k"] <= K, (M, N, K, q)
+            blk = (slice(q["m0"] // 16, (q["m0"] + q["m"]) // 16), slice(q["n0"] // 16, (q["n0"] + q["n"]) // 16))
+            cover[blk] += q["k"]
+            first[blk] += q["k0"] == 0
+            if q["variant"] != frag:
+                sub = G.make_desc(q["m"], q["n"], q["k"], a_layout=layouts[case & 1], b_layout=layouts[(case >> 1) & 1],
+                                  d_layout=layouts[(case >> 2) & 1], c_layout=layouts[(case >> 2) & 1], d_type=dt,
+                                  lda=desc.lda or (K if case & 1 else M), batch=1 + case % 3)
+                assert q["k"] % 64 == 0 and G.variant_supports(sub, q["variant"]), (M, N, K, q)
+                bm, bn = vs[q["variant"] - 1]["block"][:2]
+                tm, tn = (bn, bm) if (case >> 2) & 1 else (bm, bn)
+                if in_place:                      # whole tiles only
+                    assert q["m"] % tm == 0 and q["n"] % tn == 0, (M, N, K, q)
+            if q["k0"] > 0:                       # a k tail: Float32 D only, over the part of D its body covered
+                assert dt == np.float32 and q["variant"] == frag and q["k0"] % 64 == 0 and q["k0"] + q["k"] == K
+        assert cover.min() >= K, (M, N, K, in_place, parts)
+        if in_place:
+            assert first.min() == 1 and first.max() == 1 and cover.max() == K, (M, N, K, parts)
+        forced = G.make_desc(M, N, K, variant=frag)
+        assert [q["variant"] for q in G.plan(forced)] == [frag]
+    assert cut >= 30      # the sweep does exercise cut-up plans
+    d = G.make_desc(2000, 2000, 1984, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
+    assert len(G.plan(d)) == 1 and G.plan(d)[0]["variant"] != frag           # edge tiles shifted, K whole
+    d = G.make_desc(2000, 2000, 2000, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
+    assert [q["variant"] for q in G.plan(d)] == [frag]                        # K tail: rounding points must not move
 
 
 def test_variant_table_and_selection(miw):
