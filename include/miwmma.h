@@ -203,15 +203,17 @@ typedef struct miw_gemm_variant_info {
                            lds_bytes is then the largest ring over the operand layouts */
 } miw_gemm_variant_info;
 int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
-/* *supported = 1 when `variant` (1..count) can run this descriptor (tile divisibility, leading
-   dimensions, operand layouts, accumulate type; pointers are assumed 16-byte aligned), else 0. */
+/* *supported = 1 when `variant` (1..count) can run this descriptor (M and N of at least one tile,
+   K a multiple of 64, leading dimensions, operand layouts, accumulate type; pointers are assumed
+   16-byte aligned and C and D apart), else 0. */
 int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *supported);
 /* Variant of a single launch of this descriptor (what miw_gemm runs unless miw_gemm_plan
    cuts the problem up): the one with the shortest estimated duration
    (rounds of workgroups over the CUs, C and D traffic, and the K loop at each kernel's measured
    pace per 64 k-values) among those that can run it. */
 int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant);
-/* The launches miw_gemm makes for this descriptor.  The LDS-tiled kernels take any M and N of
+/* The launches miw_gemm makes for this descriptor (no counterpart in the reference, whose GEMM
+   would be the caller's own kernel over docs/src/device/wmma.md:51-52).  The LDS-tiled kernels take any M and N of
    at least one tile (multiples of 16, as everywhere): where the tile does not divide an extent
    the last tile is shifted back so that it ends at the edge and overlaps its neighbour; both
    workgroups compute the overlap from the same operands in the same order and store equal

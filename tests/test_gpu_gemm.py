@@ -301,7 +301,8 @@ def test_ragged_sizes_cut_into_tiled_parts_exact_on_integers(gpu, orc, al, bl, c
                                        (592, 656, 2064, dict(alpha=-2.0, beta=0.5)),
                                        (2064, 80, 1024, dict(d_type=orc.F16, c_type=orc.F16)),   # narrow: two windows over n
                                        (80, 2064, 1024, dict(use_c=0)),
-                                       (1088, 1088, 1040, dict(batch=2))]):          # only k ragged, batched
+                                       (1088, 1088, 1040, dict(batch=2)),            # only k ragged, batched
+                                       (336, 272, 192, dict(batch=3, beta=-1.0))]):  # edge tiles shifted in every problem of a batch
         pad = 8 * (n % 3)
         g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl,
                          lda=(K if al == orc.ROW else M) + pad, ldd=(N if dl == orc.ROW else M) + 2 * pad, **kw)
