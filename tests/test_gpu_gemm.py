@@ -392,6 +392,74 @@ def test_ragged_sizes_random_data_and_in_place(gpu, orc):
         assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32, (M, N, K)
 
 
+def test_seeded_sweep_over_ragged_sizes(gpu, orc):
+    """150 seeded draws of sizes that are multiples of 16 only: chosen plans and forced variants (edge tiles
+    shifted back), every layout and type combination, scalars, batches, padding and C = D in one buffer.
+    Bit-exact on integer inputs, against float64 on random ones; padding beyond D's extent stays untouched."""
+    rng = np.random.default_rng(77)
+    vs = _variants(gpu)
+    ran = cut = forced = inplace = 0
+    while ran < 150:
+        M, N = 16 * int(rng.integers(1, 60)), 16 * int(rng.integers(1, 60))
+        K = 16 * int(rng.integers(1, 40)) if rng.random() < 0.4 else 64 * int(rng.integers(1, 10))
+        al, bl, dl = (int(rng.integers(0, 2)) for _ in range(3))
+        cl = dl if rng.random() < 0.8 else 1 - dl
+        alpha = 1.0 if rng.random() < 0.6 else float(rng.choice([0.5, -2.0]))
+        beta = float(rng.choice([1.0, 0.0, -0.5, 2.0]))
+        use_c = int(rng.random() < 0.85)
+        batch = int(rng.choice([1, 1, 2, 3]))
+        ct, dt = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        pad = int(rng.choice([0, 0, 8, 16]))
+        in_place = bool(use_c and ct == dt and cl == dl and rng.random() < 0.2)
+        variant = int(rng.choice([v["id"] for v in vs[:-1]])) if rng.random() < 0.4 else 0
+        ints = rng.random() < 0.6
+        seed = int(rng.integers(0, 10000))
+        g0 = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=ct, d_type=dt).resolved()
+        g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=ct, d_type=dt,
+                         alpha=alpha, beta=beta, use_c=use_c, batch=batch, lda=g0.lda + pad, ldb=g0.ldb + pad,
+                         ldc=(g0.ldd if in_place else g0.ldc) + pad, ldd=g0.ldd + pad)
+        gr = g.resolved()
+        desc = gpu.GEMM.make_desc(M, N, K, a_layout=_W(gpu, al), b_layout=_W(gpu, bl), c_layout=_W(gpu, cl),
+                                  d_layout=_W(gpu, dl), c_type=orc.np_dtype(ct), d_type=orc.np_dtype(dt), alpha=alpha,
+                                  beta=beta, use_c=bool(use_c), batch=batch, lda=gr.lda, ldb=gr.ldb, ldc=gr.ldc, ldd=gr.ldd,
+                                  stride_a=gr.stride_a, stride_b=gr.stride_b, stride_c=gr.stride_c, stride_d=gr.stride_d,
+                                  variant=variant)
+        if variant and not gpu.GEMM.variant_supports(desc, variant):
+            continue
+        A, B, C = _inputs(orc, g, seed, ints=ints)
+        dA, dB = gpu.DeviceArray(A), gpu.DeviceArray(B)
+        if in_place:
+            dD = gpu.DeviceArray(C.copy())
+            dC = dD
+        else:
+            dD = gpu.DeviceArray(np.full(gr.stride_d * batch, 7.0, dtype=orc.np_dtype(dt)))
+            dC = gpu.DeviceArray(C) if use_c else None
+        case = (M, N, K, al, bl, cl, dl, ct, dt, alpha, beta, use_c, batch, pad, variant, in_place, ints)
+        if variant and in_place and (M % vs[variant - 1]["block"][dl == orc.ROW] or N % vs[variant - 1]["block"][dl != orc.ROW]):
+            with pytest.raises(gpu.MIWError):          # overlapping edge tiles are refused when C and D are one buffer
+                gpu.GEMM.gemm(dA, dB, dC, dD, desc)
+            continue
+        gpu.GEMM.gemm(dA, dB, dC, dD, desc)
+        gpu.synchronize()
+        D = dD.to_host()
+        ran += 1
+        forced += variant != 0
+        inplace += in_place
+        cut += variant == 0 and len(gpu.GEMM.plan(desc, in_place)) > 1
+        if ints:
+            want = orc.gemm(g, A, B, C)
+            other, inner = (M, N) if dl == orc.ROW else (N, M)
+            for bt in range(batch):
+                got = D[bt * gr.stride_d: bt * gr.stride_d + gr.ldd * other].reshape(other, gr.ldd)
+                exp = want[bt * gr.stride_d: bt * gr.stride_d + gr.ldd * other].reshape(other, gr.ldd)
+                assert np.array_equal(got[:, :inner], exp[:, :inner]), case
+                assert in_place or np.all(got[:, inner:] == 7.0), case
+        else:
+            err = orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C))
+            assert err <= (TIGHT_F32 if dt == orc.F32 else 6e-4), (case, err)
+    assert cut >= 5 and forced >= 30 and inplace >= 5, (cut, forced, inplace)
+
+
 def test_tiled_with_padded_leading_dimensions_and_batch(gpu, orc):
     g = orc.GemmDesc(M=128, N=128, K=192, lda=136, ldb=200, ldc=132, ldd=144, batch=5, a_layout=orc.COL, b_layout=orc.COL)
     A, B, C = _inputs(orc, g, 41)
