@@ -290,14 +290,17 @@ struct gemm_part {
     long m0, n0, k0;  // where the part sits in the caller's problem
 };
 
-// The fragment-op kernel: every wavefront walks K alone, 16 k-values per step, straight from global memory.
+// The fragment-op kernels.  Up to 64 k-values with C laid out as D: the short-K kernel, which moves C
+// and D at copy speed.  Otherwise every wavefront walks K alone, 16 k-values per step, straight
+// from global memory.
 double estimate_fragops_us(const miw::gemm_params &p, int c_type, int d_type)
 {
     const double mn = (double)p.M * (double)p.N * (double)p.batch;
+    const double cd_bytes = mn * (double)(dtype_size(d_type) + (p.use_c ? dtype_size(c_type) : 0));
+    const double flop = 2.0 * mn * (double)p.K;
+    if (p.K <= 64 && (!p.use_c || p.c_row == p.d_row)) return std::max(6.5, 3.0 + std::max(cd_bytes / 5.5e6, flop / 75e6));
     const double walk = 0.45 * (double)(p.K / 16);
-    const double flops = 2.0 * mn * (double)p.K / 45e6;
-    const double bytes = mn * (double)(dtype_size(d_type) + (p.use_c ? dtype_size(c_type) : 0)) / 2.0e6;
-    return 5.0 + std::max(walk, std::max(flops, bytes));
+    return 5.0 + std::max(walk, std::max(flop / 45e6, cd_bytes / 2.0e6));
 }
 
 miw::gemm_params sub_block(const miw::gemm_params &p, int c_type, int d_type, long m0, long m, long n0, long n)

@@ -291,6 +291,154 @@ __global__ __launch_bounds__(256) void k_gemm_fragops(gemm_params p)
     store_d<config<16, 16, 16, DT>, DT>(Dt, d, p.ldd, ld);
 }
 
+// ---------------------------------------------------------------------------
+// The same chain of mma calls for a short K (16 to 64 k-values) and Float32 accumulation, where
+// the run time is the traffic of C and D: the last k-values of a problem whose K no LDS tile
+// divides (with D as the C operand), or a rank-16..64 update.  One workgroup of four wavefronts
+// per 64 x 64 block of D in canonical form (P = X*Y with i contiguous in P: X = A, Y = B for a
+// column-major D, X = B^T, Y = A^T for a row-major one); a wavefront owns 16 columns and chains the
+// mma calls of its four 16 x 16 tiles.  The accumulator layout would read and write 64 contiguous
+// bytes per column and instruction, so the sums go through a private piece of LDS (68 floats per
+// column: the 16 lanes that store, and later read, one 16-byte piece of 16 different columns or
+// rows hit 16 different groups of four banks) and C and D move as 256 contiguous bytes per column.
+// C must be laid out as D (the caller's other case runs on k_gemm_fragops).
+struct shortk_params {
+    const half_t *X, *Y;
+    const void *C;
+    void *D;
+    long I, J, K;
+    long ldx, ldy, ldc, ldd;
+    long sx, sy, sc, sd;
+    int x_row, y_row;  // X stored with k contiguous; Y stored with j contiguous
+    int use_c;
+    float alpha, beta;
+};
+
+template <class CT, class DT>
+__global__ __launch_bounds__(256) void k_gemm_shortk(shortk_params p)
+{
+    constexpr int PITCH = 68;   // floats per staged column of sums
+    constexpr int KP = 64 + 8;  // halves per staged operand row (k contiguous)
+    __shared__ __attribute__((aligned(16))) float stage[4][16 * PITCH];
+    __shared__ __attribute__((aligned(16))) half_t xs[64 * KP], ys[64 * KP];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int q = lane >> 4, r = lane & 15;
+    const long blocks_i = (p.I + 63) / 64;
+    const long i0 = (long)(blockIdx.x % blocks_i) * 64, jb = (long)(blockIdx.x / blocks_i) * 64, j0 = jb + 16 * wave;
+    const long bt = blockIdx.y;
+    const half_t *X = p.X + bt * p.sx;
+    const half_t *Y = p.Y + bt * p.sy;
+    const CT *C = (const CT *)p.C + bt * p.sc;
+    DT *D = (DT *)p.D + bt * p.sd;
+
+    // Both operand blocks (64 rows of X, 64 columns of Y, all of K) go to LDS with k contiguous, in
+    // 16-byte pieces along whichever dimension is contiguous in memory; rows past the edge repeat the last one.
+    const int K = (int)p.K, kc = K / 8;
+    auto stage_operand = [&](half_t *dst, const half_t *src, long ld, bool k_contiguous, long first, long extent) {
+        if (k_contiguous) {
+            for (int c = tid; c < 64 * kc; c += 256) {
+                const int row = c / kc, piece = c % kc;
+                const long g = min(first + row, extent - 1);
+                *(half8_t *)(dst + row * KP + piece * 8) = *(const half8_t *)(src + g * ld + piece * 8);
+            }
+        } else {
+            for (int c = tid; c < K * 8; c += 256) {
+                const int k = c >> 3, piece = c & 7;
+                const long g = min(first + piece * 8, extent - 8);
+                const half8_t v = *(const half8_t *)(src + (long)k * ld + g);
+                const int row0 = (int)(g - first);
+#pragma unroll
+                for (int e = 0; e < 8; e++) dst[(row0 + e) * KP + k] = v[e];
+            }
+        }
+    };
+    stage_operand(xs, X, p.ldx, p.x_row != 0, i0, p.I);
+    stage_operand(ys, Y, p.ldy, p.y_row == 0, jb, p.J);
+    __syncthreads();
+    if (j0 >= p.J) return;  // (wavefront-uniform; no barrier below)
+
+    float4_t acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        const half4_t y = *(const half4_t *)(ys + (16 * wave + r) * KP + k0 + 4 * q);  // x[e] = Y[k0 + 4q + e][j0 + r]
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const half4_t x = *(const half4_t *)(xs + (16 * t + r) * KP + k0 + 4 * q);  // x[e] = X[i0 + 16t + r][k0 + 4q + e]
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(x, y, acc[t], 0, 0, 0);
+        }
+    }
+    // accumulator layout (rows 16t + 4q .. + 3 of column r) -> LDS, 64 rows of a column contiguous
+    float *mine = stage[wave];
+#pragma unroll
+    for (int t = 0; t < 4; t++) *(float4_t *)(mine + r * PITCH + 16 * t + 4 * q) = acc[t];
+    // (LDS operations of one wavefront complete in order)
+#pragma unroll
+    for (int n = 0; n < 4; n++) {
+        const int c = 4 * n + (lane >> 4), m = lane & 15;  // column of the wavefront's 16, 4-row piece of the 64 rows
+        const long i = i0 + 4 * m, j = j0 + c;
+        if (i >= p.I || j >= p.J) continue;
+        float4_t v = *(const float4_t *)(mine + c * PITCH + 4 * m);
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] *= p.alpha;
+        if (p.use_c) {
+            float4_t cv;
+            if constexpr (__is_same(CT, float)) {
+                cv = *(const float4_t *)(C + j * p.ldc + i);
+            } else {
+                const half4_t h = *(const half4_t *)(C + j * p.ldc + i);
+                cv = float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, cv[e], v[e]);
+        }
+        if constexpr (__is_same(DT, float)) {
+            *(float4_t *)(D + j * p.ldd + i) = v;
+        } else {
+            const half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+            *(half4_t *)(D + j * p.ldd + i) = h;
+        }
+    }
+}
+
+// Can k_gemm_shortk run this problem?  Float32 accumulation, K up to 64, C laid out as D, and every
+// operand aligned for 16-byte accesses.
+static bool shortk_fits(const gemm_params &p, int c_type, int d_type, bool f16acc)
+{
+    if (f16acc || p.K > 64) return false;
+    if (((uintptr_t)p.A & 15) || ((uintptr_t)p.B & 15) || p.lda % 8 || p.ldb % 8 || p.sa % 8 || p.sb % 8) return false;
+    if (p.use_c && p.c_row != p.d_row) return false;
+    const long dper = d_type == 0 ? 8 : 4, cper = c_type == 0 ? 8 : 4;  // elements per 16 bytes
+    if (((uintptr_t)p.D & 15) || p.ldd % dper || p.sd % dper) return false;
+    if (p.use_c && (((uintptr_t)p.C & 15) || p.ldc % cper || p.sc % cper)) return false;
+    const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
+    return ((I + 63) / 64) * ((J + 63) / 64) < (1l << 31);
+}
+
+static hipError_t launch_gemm_shortk(const gemm_params &g, int c_type, int d_type, hipStream_t s)
+{
+    shortk_params p;
+    if (!g.d_row) {
+        p.X = g.A; p.Y = g.B; p.I = g.M; p.J = g.N;
+        p.ldx = g.lda; p.ldy = g.ldb; p.sx = g.sa; p.sy = g.sb;
+        p.x_row = g.a_row; p.y_row = g.b_row;
+    } else {
+        // D^T = B^T * A^T: X[i][k] = B[k][i], Y[k][j] = A[j][k]
+        p.X = g.B; p.Y = g.A; p.I = g.N; p.J = g.M;
+        p.ldx = g.ldb; p.ldy = g.lda; p.sx = g.sb; p.sy = g.sa;
+        p.x_row = !g.b_row; p.y_row = !g.a_row;
+    }
+    p.C = g.C; p.D = g.D; p.K = g.K;
+    p.ldc = g.ldc; p.ldd = g.ldd; p.sc = g.sc; p.sd = g.sd;
+    p.use_c = g.use_c; p.alpha = g.alpha; p.beta = g.beta;
+    dim3 grid((unsigned)(((p.I + 63) / 64) * ((p.J + 63) / 64)), (unsigned)g.batch);
+    if (c_type == 0 && d_type == 0) hipLaunchKernelGGL((k_gemm_shortk<half_t, half_t>), grid, dim3(256), 0, s, p);
+    else if (c_type == 0 && d_type == 1) hipLaunchKernelGGL((k_gemm_shortk<half_t, float>), grid, dim3(256), 0, s, p);
+    else if (c_type == 1 && d_type == 0) hipLaunchKernelGGL((k_gemm_shortk<float, half_t>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((k_gemm_shortk<float, float>), grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------ launchers ----
 
 hipError_t launch_frag_load(int use, int dtype, int row_major, int as_mode, const void *addr, long stride, void *img,
@@ -365,6 +513,7 @@ hipError_t launch_wmma_mac(int c_type, int d_type, const void *A, const void *B,
 
 hipError_t launch_gemm_fragops(const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s)
 {
+    if (shortk_fits(p, c_type, d_type, f16acc)) return launch_gemm_shortk(p, c_type, d_type, s);
     const long tiles = (p.M / 16) * (p.N / 16);
     dim3 grid((unsigned)((tiles + 3) / 4), (unsigned)p.batch);
     if (f16acc) {

@@ -460,6 +460,46 @@ def test_seeded_sweep_over_ragged_sizes(gpu, orc):
     assert cut >= 5 and forced >= 30 and inplace >= 5, (cut, forced, inplace)
 
 
+@pytest.mark.parametrize("al,bl,dl", itertools.product((0, 1), repeat=3))
+def test_short_k_kernel_of_the_fragment_op_path(gpu, orc, al, bl, dl):
+    """K of 16 to 64 on the fragment-op variant runs a kernel of its own (operands staged through LDS, C
+    and D moved in whole columns): bit-exact on integers for every layout, type combination, ragged
+    block edges, batches, scalars and C = D; leading dimensions that are no multiple of 16 bytes take
+    the one-wavefront-per-tile kernel and must give the same bits."""
+    frag = _variants(gpu)[-1]["id"]
+    n = 0
+    for K in (16, 32, 48, 64):
+        for M, N in ((64, 64), (80, 208), (272, 48), (16, 16)):
+            ct, dt = (n >> 1) & 1, n & 1
+            n += 1
+            g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, c_type=ct, d_type=dt,
+                             alpha=(1.0, -2.0, 0.5)[n % 3], beta=(1.0, 0.5, -1.0)[n % 3], batch=1 + n % 2,
+                             ldd=(N if dl == orc.ROW else M) + 8 * (n % 2))
+            A, B, C = _inputs(orc, g, 1500 + n, ints=True)
+            def check(gd, Ad):
+                want = orc.gemm(gd, Ad, B, C)
+                D = _run(gpu, orc, gd, Ad, B, C, variant=frag, prefill=7.0)
+                gr = gd.resolved()
+                other, inner = (M, N) if dl == orc.ROW else (N, M)
+                for bt in range(max(gr.batch, 1)):
+                    got = D[bt * gr.stride_d: bt * gr.stride_d + gr.ldd * other].reshape(other, gr.ldd)
+                    exp = want[bt * gr.stride_d: bt * gr.stride_d + gr.ldd * other].reshape(other, gr.ldd)
+                    assert np.array_equal(got[:, :inner], exp[:, :inner]), (M, N, K, al, bl, dl, ct, dt, gr.lda)
+                    assert np.all(got[:, inner:] == 7.0)
+            check(g, A)
+            # the same problem with a leading dimension of A that is not a multiple of 8 elements
+            g2 = orc.GemmDesc(**{**g.__dict__, "lda": (K if al == orc.ROW else M) + 2})
+            check(g2, _inputs(orc, g2, 1500 + n, ints=True)[0])
+    # in place, random data
+    g = orc.GemmDesc(M=208, N=80, K=48, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, beta=0.5)
+    A, B, C = _inputs(orc, g, 1590)
+    dA, dB, dD = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(C.copy())
+    gpu.GEMM.gemm(dA, dB, dD, dD, gpu.GEMM.make_desc(208, 80, 48, a_layout=_W(gpu, al), b_layout=_W(gpu, bl),
+                                                     c_layout=_W(gpu, dl), d_layout=_W(gpu, dl), beta=0.5, variant=frag))
+    gpu.synchronize()
+    assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+
+
 def test_tiled_with_padded_leading_dimensions_and_batch(gpu, orc):
     g = orc.GemmDesc(M=128, N=128, K=192, lda=136, ldb=200, ldc=132, ldd=144, batch=5, a_layout=orc.COL, b_layout=orc.COL)
     A, B, C = _inputs(orc, g, 41)
