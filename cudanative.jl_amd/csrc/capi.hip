@@ -299,7 +299,8 @@ double estimate_fragops_us(const miw::gemm_params &p, int c_type, int d_type)
     const double cd_bytes = mn * (double)(dtype_size(d_type) + (p.use_c ? dtype_size(c_type) : 0));
     const double flop = 2.0 * mn * (double)p.K;
     if (p.K <= 64 && (!p.use_c || p.c_row == p.d_row)) return std::max(6.5, 3.0 + std::max(cd_bytes / 5.5e6, flop / 75e6));
-    const double walk = 0.45 * (double)(p.K / 16);
+    const int split = miw::fragops_ksplit(p, false);  // few tiles, long K: several wavefronts share a tile's K loop
+    const double walk = 0.45 * (double)(p.K / 16) / split + (split > 1 ? 2.0 : 0.0);
     return 5.0 + std::max(walk, std::max(flop / 45e6, cd_bytes / 2.0e6));
 }
 

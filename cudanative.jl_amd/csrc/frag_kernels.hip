@@ -439,6 +439,79 @@ static hipError_t launch_gemm_shortk(const gemm_params &g, int c_type, int d_typ
     return hipGetLastError();
 }
 
+// The same chain for problems with few output tiles and a long K (a thin D: 16 to 48 rows or
+// columns): S wavefronts of one workgroup share a tile, wavefront w takes k-steps w, w + S, ...,
+// and wavefront 0 adds the S partial sums in wavefront order (through LDS) before the epilogue.
+// Float32 accumulation only (the Float16 chain rounds after every step, in order).  The result
+// does not depend on timing; it differs from k_gemm_fragops' in the order of the Float32 additions.
+template <class CT, class DT>
+__global__ __launch_bounds__(1024) void k_gemm_fragops_ksplit(gemm_params p)
+{
+    using cfg32 = config<16, 16, 16, float>;
+    extern __shared__ __attribute__((aligned(16))) float partial[];  // [wavefront][lane][4]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, S = blockDim.x >> 6;
+    const long tiles_m = p.M / 16;
+    const long tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    const long bt = blockIdx.y;
+    const half_t *A = p.A + bt * p.sa;
+    const half_t *B = p.B + bt * p.sb;
+    const CT *C = (const CT *)p.C + bt * p.sc;
+    DT *D = (DT *)p.D + bt * p.sd;
+    const layout lc = p.c_row ? layout::row_major : layout::col_major;
+    const layout ld = p.d_row ? layout::row_major : layout::col_major;
+
+    fragment<accumulator, 16, 16, 16, float, layout::unspecified> acc = fill_c<cfg32, float>(0.f);
+    for (long k0 = 16l * wave; k0 < p.K; k0 += 16l * S) {
+        const half_t *At = A + (p.a_row ? tm * 16 * p.lda + k0 : tm * 16 + k0 * p.lda);
+        const half_t *Bt = B + (p.b_row ? k0 * p.ldb + tn * 16 : k0 + tn * 16 * p.ldb);
+        fragment<matrix_a, 16, 16, 16, half_t, layout::col_major> a;
+        fragment<matrix_b, 16, 16, 16, half_t, layout::col_major> b;
+        if (p.a_row) {
+            auto t = load_a<cfg32, layout::row_major>(At, p.lda);
+            for (int i = 0; i < 4; i++) a.x[i] = t.x[i];
+        } else {
+            a = load_a<cfg32, layout::col_major>(At, p.lda);
+        }
+        if (p.b_row) {
+            auto t = load_b<cfg32, layout::row_major>(Bt, p.ldb);
+            for (int i = 0; i < 4; i++) b.x[i] = t.x[i];
+        } else {
+            b = load_b<cfg32, layout::col_major>(Bt, p.ldb);
+        }
+        acc = mma<cfg32>(a, b, acc);
+    }
+    if (wave) *(float4_t *)(partial + (wave * 64 + lane) * 4) = float4_t{acc.x[0], acc.x[1], acc.x[2], acc.x[3]};
+    __syncthreads();
+    if (wave) return;
+    for (int w = 1; w < S; w++) {
+        const float4_t v = *(const float4_t *)(partial + (w * 64 + lane) * 4);
+        for (int i = 0; i < 4; i++) acc.x[i] += v[i];
+    }
+    const CT *Ct = C + tile_offset(lc, (int)(tm * 16), 0, p.ldc) + tile_offset(lc, 0, (int)(tn * 16), p.ldc);
+    DT *Dt = D + tile_offset(ld, (int)(tm * 16), 0, p.ldd) + tile_offset(ld, 0, (int)(tn * 16), p.ldd);
+    fragment<accumulator, 16, 16, 16, DT, layout::unspecified> d;
+    fragment<accumulator, 16, 16, 16, CT, layout::unspecified> cf;
+    if (p.use_c) cf = load_c<cfg32, CT>(Ct, p.ldc, lc);
+    for (int i = 0; i < 4; i++) {
+        float v = p.alpha * acc.x[i];
+        if (p.use_c) v = __builtin_fmaf(p.beta, (float)cf.x[i], v);
+        d.x[i] = (DT)v;
+    }
+    store_d<config<16, 16, 16, DT>, DT>(Dt, d, p.ldd, ld);
+}
+
+// Wavefronts per tile k_gemm_fragops_ksplit would use for this problem, or 1 for the
+// one-wavefront-per-tile kernel: few tiles (fewer than 32 wavefronts per CU of a 256-CU part even
+// with the split) and at least four k-steps per wavefront.
+int fragops_ksplit(const gemm_params &p, bool f16acc)
+{
+    if (f16acc) return 1;
+    const long tiles = (p.M / 16) * (p.N / 16) * p.batch;
+    int s = 16;
+    while (s > 1 && (tiles * s > 8192 || p.K / (16l * s) < 4)) s >>= 1;
+    return s >= 4 ? s : 1;
+}
+
 // ------------------------------------------------------------ launchers ----
 
 hipError_t launch_frag_load(int use, int dtype, int row_major, int as_mode, const void *addr, long stride, void *img,
@@ -514,6 +587,15 @@ hipError_t launch_wmma_mac(int c_type, int d_type, const void *A, const void *B,
 hipError_t launch_gemm_fragops(const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s)
 {
     if (shortk_fits(p, c_type, d_type, f16acc)) return launch_gemm_shortk(p, c_type, d_type, s);
+    if (const int split = fragops_ksplit(p, f16acc); split > 1) {
+        dim3 grid((unsigned)((p.M / 16) * (p.N / 16)), (unsigned)p.batch), block((unsigned)(64 * split));
+        const size_t lds = (size_t)split * 64 * 4 * sizeof(float);
+        if (c_type == 0 && d_type == 0) hipLaunchKernelGGL((k_gemm_fragops_ksplit<half_t, half_t>), grid, block, lds, s, p);
+        else if (c_type == 0 && d_type == 1) hipLaunchKernelGGL((k_gemm_fragops_ksplit<half_t, float>), grid, block, lds, s, p);
+        else if (c_type == 1 && d_type == 0) hipLaunchKernelGGL((k_gemm_fragops_ksplit<float, half_t>), grid, block, lds, s, p);
+        else hipLaunchKernelGGL((k_gemm_fragops_ksplit<float, float>), grid, block, lds, s, p);
+        return hipGetLastError();
+    }
     const long tiles = (p.M / 16) * (p.N / 16);
     dim3 grid((unsigned)((tiles + 3) / 4), (unsigned)p.batch);
     if (f16acc) {

@@ -34,6 +34,8 @@ hipError_t launch_wmma_mac(int c_type, int d_type, const void *A, const void *B,
                            long ldb, long ldc, long ldd, int a_row, int b_row, int c_row, int d_row, int use_c,
                            int shared, float alpha, float beta, hipStream_t s);
 hipError_t launch_gemm_fragops(const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s);
+// Wavefronts that share one 16x16 tile's K loop in the fragment-op kernel launch_gemm_fragops picks (1: none).
+int fragops_ksplit(const gemm_params &p, bool f16acc);
 hipError_t launch_dummy_store(float *ptr, int threads, hipStream_t s);
 const void *frag_kernel_symbol(const char *name);
 int frag_kernel_count();
