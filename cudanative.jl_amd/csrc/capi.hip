@@ -919,7 +919,7 @@ int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void
     }
     if (splits == 0)
         return fail(MIW_ERR_UNSUPPORTED,
-                    "gemm_splitk: needs K divisible by 64 * splits, M and N divisible by an LDS tile (64 at least), "
+                    "gemm_splitk: needs K divisible by 64 * splits, M and N of at least one LDS tile (64), "
                     "16-byte aligned operands and leading dimensions");
     out->full = p;
     out->splits = splits;

@@ -243,7 +243,7 @@ int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk);
    (splits * m * n * 4 bytes, 16-byte aligned, contents on entry irrelevant), and a second kernel
    adds the slices in order: D = alpha * sum_s A_s*B_s + beta*C.  The result does not depend on
    timing; it differs from miw_gemm's by the rounding of one Float32 sum per slice.  Float32
-   accumulation, batch 1, desc.variant 0, M and N divisible by an LDS tile.  splits = 0 chooses
+   accumulation, batch 1, desc.variant 0, M and N of at least one LDS tile (64).  splits = 0 chooses
    the slice count with the shortest estimated duration (both kernels and the workspace traffic
    counted).  One slice, asked for or chosen, is the plain launch of miw_gemm: no workspace
    (0 bytes, `workspace` may be null) and no second kernel.  miw_gemm_splitk_workspace reports
