@@ -5,6 +5,8 @@
 #include "kernels.hpp"
 #include "miwmma_fragment.hpp"
 
+#include <type_traits>
+
 namespace miw {
 
 using cfg_f32 = config<16, 16, 16, float>;
@@ -439,19 +441,23 @@ static hipError_t launch_gemm_shortk(const gemm_params &g, int c_type, int d_typ
     return hipGetLastError();
 }
 
-// The same chain for problems with few output tiles and a long K (a thin D: 16 to 48 rows or
-// columns): S wavefronts of one workgroup share a tile, wavefront w takes k-steps w, w + S, ...,
-// and wavefront 0 adds the S partial sums in wavefront order (through LDS) before the epilogue.
+// The same chain for problems with few output tiles and a long K: S wavefronts of one workgroup
+// share the K loop, wavefront w takes k-steps w, w + S, ..., and wavefront 0 adds the S partial sums
+// in wavefront order (through LDS) before the epilogue.  A thin D (16 to 64 rows, or columns) is
+// taken T tiles at a time, all tiles of the thin dimension by one workgroup, so that the fragment
+// of the long operand is loaded once for them; otherwise T = 1 and a workgroup owns one tile.
 // Float32 accumulation only (the Float16 chain rounds after every step, in order).  The result
 // does not depend on timing; it differs from k_gemm_fragops' in the order of the Float32 additions.
-template <class CT, class DT>
-__global__ __launch_bounds__(1024) void k_gemm_fragops_ksplit(gemm_params p)
+template <class CT, class DT, int T>
+__global__ __launch_bounds__(1024) void k_gemm_fragops_ksplit(gemm_params p, int thin_m)
 {
     using cfg32 = config<16, 16, 16, float>;
-    extern __shared__ __attribute__((aligned(16))) float partial[];  // [wavefront][lane][4]
+    extern __shared__ __attribute__((aligned(16))) float partial[];  // [wavefront][tile][lane][4]
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, S = blockDim.x >> 6;
     const long tiles_m = p.M / 16;
-    const long tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    // T == 1: one tile (tm, tn).  T > 1: tiles (t, tn), t < T, of a D with 16 T rows (thin_m), or (tm, t) of one with 16 T columns.
+    const long tm0 = T > 1 ? (thin_m ? 0 : blockIdx.x) : blockIdx.x % tiles_m;
+    const long tn0 = T > 1 ? (thin_m ? blockIdx.x : 0) : blockIdx.x / tiles_m;
     const long bt = blockIdx.y;
     const half_t *A = p.A + bt * p.sa;
     const half_t *B = p.B + bt * p.sb;
@@ -459,45 +465,71 @@ __global__ __launch_bounds__(1024) void k_gemm_fragops_ksplit(gemm_params p)
     DT *D = (DT *)p.D + bt * p.sd;
     const layout lc = p.c_row ? layout::row_major : layout::col_major;
     const layout ld = p.d_row ? layout::row_major : layout::col_major;
-
-    fragment<accumulator, 16, 16, 16, float, layout::unspecified> acc = fill_c<cfg32, float>(0.f);
-    for (long k0 = 16l * wave; k0 < p.K; k0 += 16l * S) {
-        const half_t *At = A + (p.a_row ? tm * 16 * p.lda + k0 : tm * 16 + k0 * p.lda);
-        const half_t *Bt = B + (p.b_row ? k0 * p.ldb + tn * 16 : k0 + tn * 16 * p.ldb);
-        fragment<matrix_a, 16, 16, 16, half_t, layout::col_major> a;
-        fragment<matrix_b, 16, 16, 16, half_t, layout::col_major> b;
-        if (p.a_row) {
-            auto t = load_a<cfg32, layout::row_major>(At, p.lda);
-            for (int i = 0; i < 4; i++) a.x[i] = t.x[i];
-        } else {
-            a = load_a<cfg32, layout::col_major>(At, p.lda);
+    fragment<accumulator, 16, 16, 16, float, layout::unspecified> acc[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) acc[t] = fill_c<cfg32, float>(0.f);
+    // The K loop, once per combination of operand layouts (they are uniform over the grid): the
+    // loads of a fragment are 8 contiguous bytes per lane where k is contiguous.
+    auto walk = [&]<bool AR, bool BR>(std::bool_constant<AR>, std::bool_constant<BR>) {
+        constexpr layout la = AR ? layout::row_major : layout::col_major, lb = BR ? layout::row_major : layout::col_major;
+        for (long k0 = 16l * wave; k0 < p.K; k0 += 16l * S) {
+            if (T > 1 && !thin_m) {
+                const auto a = load_a<cfg32, la>(A + tile_offset(la, (int)(tm0 * 16), 0, p.lda) + tile_offset(la, 0, (int)k0, p.lda), p.lda);
+#pragma unroll
+                for (int t = 0; t < T; t++) {
+                    const auto b = load_b<cfg32, lb>(B + tile_offset(lb, (int)k0, 0, p.ldb) + tile_offset(lb, 0, t * 16, p.ldb), p.ldb);
+                    acc[t] = mma<cfg32>(a, b, acc[t]);
+                }
+            } else {
+                const auto b = load_b<cfg32, lb>(B + tile_offset(lb, (int)k0, 0, p.ldb) + tile_offset(lb, 0, (int)(tn0 * 16), p.ldb), p.ldb);
+#pragma unroll
+                for (int t = 0; t < T; t++) {
+                    const auto a = load_a<cfg32, la>(A + tile_offset(la, (int)((tm0 + t) * 16), 0, p.lda) + tile_offset(la, 0, (int)k0, p.lda), p.lda);
+                    acc[t] = mma<cfg32>(a, b, acc[t]);
+                }
+            }
         }
-        if (p.b_row) {
-            auto t = load_b<cfg32, layout::row_major>(Bt, p.ldb);
-            for (int i = 0; i < 4; i++) b.x[i] = t.x[i];
-        } else {
-            b = load_b<cfg32, layout::col_major>(Bt, p.ldb);
-        }
-        acc = mma<cfg32>(a, b, acc);
+    };
+    if (p.a_row && p.b_row) walk(std::true_type{}, std::true_type{});
+    else if (p.a_row) walk(std::true_type{}, std::false_type{});
+    else if (p.b_row) walk(std::false_type{}, std::true_type{});
+    else walk(std::false_type{}, std::false_type{});
+    if (wave) {
+#pragma unroll
+        for (int t = 0; t < T; t++)
+            *(float4_t *)(partial + ((wave * T + t) * 64 + lane) * 4) = float4_t{acc[t].x[0], acc[t].x[1], acc[t].x[2], acc[t].x[3]};
     }
-    if (wave) *(float4_t *)(partial + (wave * 64 + lane) * 4) = float4_t{acc.x[0], acc.x[1], acc.x[2], acc.x[3]};
     __syncthreads();
     if (wave) return;
-    for (int w = 1; w < S; w++) {
-        const float4_t v = *(const float4_t *)(partial + (w * 64 + lane) * 4);
-        for (int i = 0; i < 4; i++) acc.x[i] += v[i];
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        for (int w = 1; w < S; w++) {
+            const float4_t v = *(const float4_t *)(partial + ((w * T + t) * 64 + lane) * 4);
+            for (int i = 0; i < 4; i++) acc[t].x[i] += v[i];
+        }
+        const long tm = T > 1 && thin_m ? t : tm0, tn = T > 1 && !thin_m ? t : tn0;
+        const CT *Ct = C + tile_offset(lc, (int)(tm * 16), 0, p.ldc) + tile_offset(lc, 0, (int)(tn * 16), p.ldc);
+        DT *Dt = D + tile_offset(ld, (int)(tm * 16), 0, p.ldd) + tile_offset(ld, 0, (int)(tn * 16), p.ldd);
+        fragment<accumulator, 16, 16, 16, DT, layout::unspecified> d;
+        fragment<accumulator, 16, 16, 16, CT, layout::unspecified> cf;
+        if (p.use_c) cf = load_c<cfg32, CT>(Ct, p.ldc, lc);
+        for (int i = 0; i < 4; i++) {
+            float v = p.alpha * acc[t].x[i];
+            if (p.use_c) v = __builtin_fmaf(p.beta, (float)cf.x[i], v);
+            d.x[i] = (DT)v;
+        }
+        store_d<config<16, 16, 16, DT>, DT>(Dt, d, p.ldd, ld);
     }
-    const CT *Ct = C + tile_offset(lc, (int)(tm * 16), 0, p.ldc) + tile_offset(lc, 0, (int)(tn * 16), p.ldc);
-    DT *Dt = D + tile_offset(ld, (int)(tm * 16), 0, p.ldd) + tile_offset(ld, 0, (int)(tn * 16), p.ldd);
-    fragment<accumulator, 16, 16, 16, DT, layout::unspecified> d;
-    fragment<accumulator, 16, 16, 16, CT, layout::unspecified> cf;
-    if (p.use_c) cf = load_c<cfg32, CT>(Ct, p.ldc, lc);
-    for (int i = 0; i < 4; i++) {
-        float v = p.alpha * acc.x[i];
-        if (p.use_c) v = __builtin_fmaf(p.beta, (float)cf.x[i], v);
-        d.x[i] = (DT)v;
-    }
-    store_d<config<16, 16, 16, DT>, DT>(Dt, d, p.ldd, ld);
+}
+
+// Tiles a workgroup of k_gemm_fragops_ksplit takes together: all 2 to 4 tiles of a thin dimension where the
+// other dimension still gives 64 workgroups or more per problem, else 1.
+static int ksplit_tiles(const gemm_params &p, int *thin_m)
+{
+    const long tm = p.M / 16, tn = p.N / 16;
+    *thin_m = tm <= tn;
+    const long t = tm <= tn ? tm : tn, other = tm <= tn ? tn : tm;
+    return t >= 2 && t <= 4 && other >= 64 ? (int)t : 1;
 }
 
 // Wavefronts per tile k_gemm_fragops_ksplit would use for this problem, or 1 for the
@@ -506,9 +538,10 @@ __global__ __launch_bounds__(1024) void k_gemm_fragops_ksplit(gemm_params p)
 int fragops_ksplit(const gemm_params &p, bool f16acc)
 {
     if (f16acc) return 1;
-    const long tiles = (p.M / 16) * (p.N / 16) * p.batch;
+    int thin_m;
+    const long groups = (p.M / 16) * (p.N / 16) / ksplit_tiles(p, &thin_m) * p.batch;  // workgroups
     int s = 16;
-    while (s > 1 && (tiles * s > 8192 || p.K / (16l * s) < 4)) s >>= 1;
+    while (s > 1 && (groups * s > 8192 || p.K / (16l * s) < 4)) s >>= 1;
     return s >= 4 ? s : 1;
 }
 
@@ -588,12 +621,20 @@ hipError_t launch_gemm_fragops(const gemm_params &p, int c_type, int d_type, boo
 {
     if (shortk_fits(p, c_type, d_type, f16acc)) return launch_gemm_shortk(p, c_type, d_type, s);
     if (const int split = fragops_ksplit(p, f16acc); split > 1) {
-        dim3 grid((unsigned)((p.M / 16) * (p.N / 16)), (unsigned)p.batch), block((unsigned)(64 * split));
-        const size_t lds = (size_t)split * 64 * 4 * sizeof(float);
-        if (c_type == 0 && d_type == 0) hipLaunchKernelGGL((k_gemm_fragops_ksplit<half_t, half_t>), grid, block, lds, s, p);
-        else if (c_type == 0 && d_type == 1) hipLaunchKernelGGL((k_gemm_fragops_ksplit<half_t, float>), grid, block, lds, s, p);
-        else if (c_type == 1 && d_type == 0) hipLaunchKernelGGL((k_gemm_fragops_ksplit<float, half_t>), grid, block, lds, s, p);
-        else hipLaunchKernelGGL((k_gemm_fragops_ksplit<float, float>), grid, block, lds, s, p);
+        int thin_m;
+        const int T = ksplit_tiles(p, &thin_m);
+        dim3 grid((unsigned)((p.M / 16) * (p.N / 16) / T), (unsigned)p.batch), block((unsigned)(64 * split));
+        const size_t lds = (size_t)split * T * 64 * 4 * sizeof(float);
+        auto go = [&]<class CT, class DT>(CT, DT) {
+            if (T == 1) hipLaunchKernelGGL((k_gemm_fragops_ksplit<CT, DT, 1>), grid, block, lds, s, p, thin_m);
+            else if (T == 2) hipLaunchKernelGGL((k_gemm_fragops_ksplit<CT, DT, 2>), grid, block, lds, s, p, thin_m);
+            else if (T == 3) hipLaunchKernelGGL((k_gemm_fragops_ksplit<CT, DT, 3>), grid, block, lds, s, p, thin_m);
+            else hipLaunchKernelGGL((k_gemm_fragops_ksplit<CT, DT, 4>), grid, block, lds, s, p, thin_m);
+        };
+        if (c_type == 0 && d_type == 0) go(half_t{}, half_t{});
+        else if (c_type == 0 && d_type == 1) go(half_t{}, float{});
+        else if (c_type == 1 && d_type == 0) go(float{}, half_t{});
+        else go(float{}, float{});
         return hipGetLastError();
     }
     const long tiles = (p.M / 16) * (p.N / 16);

@@ -509,7 +509,11 @@ def test_thin_problems_share_a_tile_between_wavefronts(gpu, orc, al, bl, cl, dl)
     frag = _variants(gpu)[-1]["id"]
     for n, (M, N, K, kw) in enumerate([(16, 256, 2048, {}), (48, 64, 1024, dict(alpha=0.5, beta=-2.0)),
                                        (32, 32, 4096, dict(batch=2, c_type=orc.F16, d_type=orc.F16)),
-                                       (272, 16, 1040, dict(use_c=0, d_type=orc.F16)), (16, 16, 16384, {})]):
+                                       (272, 16, 1040, dict(use_c=0, d_type=orc.F16)), (16, 16, 16384, {}),
+                                       (272, 48, 1024, dict(beta=0.5)), (64, 272, 1040, dict(d_type=orc.F16, c_type=orc.F16)),
+                                       # all tiles of the thin dimension in one workgroup (2, 3 and 4 of them)
+                                       (32, 1024, 512, dict(beta=-1.0)), (1024, 48, 512, dict(alpha=2.0, batch=2)),
+                                       (64, 1024, 528, dict(d_type=orc.F16, c_type=orc.F16))]):
         g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl,
                          ldd=(N if dl == orc.ROW else M) + 8, **kw)
         assert [q["variant"] for q in _plan(gpu, orc, g)][-1] == frag
