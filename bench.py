@@ -111,6 +111,81 @@ def library_reference():
     print(json.dumps({"library_reference": "torch.matmul Float16 4096^3 (torch %s)" % torch.__version__, "results": out}))
 
 
+SWEEP_SHAPES = [(512, 512, 512), (1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (3072, 3072, 3072),
+                (4096, 4096, 4096), (6144, 6144, 6144), (8192, 8192, 8192), (8192, 8192, 1024), (1024, 8192, 8192),
+                (4096, 4096, 512), (4096, 4096, 16384), (2048, 8192, 4096), (8192, 1024, 4096), (256, 256, 8192),
+                (4096, 128, 4096), (128, 4096, 4096), (16, 4096, 4096), (48, 4096, 4096),
+                (4352, 4224, 4096), (4160, 4096, 4160), (4144, 4096, 4096), (4000, 4000, 4096), (4000, 4000, 4000),
+                (4096, 4096, 4112), (2000, 2000, 2000)]
+
+
+def shape_sweep(vendor):
+    """A comparison aid: Float16 operands in U[-1,1), A column-major and row-major with B column-major, over
+    SWEEP_SHAPES.  This library (Float32 C and D, D = A*B + C): the launches miw_gemm makes by itself and, for
+    a size a tile divides, every single variant that can run it, each after 0.25 s of untimed launches,
+    median of 30 event-timed launches.  vendor: torch.matmul (hipBLASLt / rocBLAS; Float16 out, no C) timed
+    over 30 back-to-back launches.  The two use different HIP runtimes, hence two invocations."""
+    out = []
+    if vendor:
+        import torch
+        for M, N, K in SWEEP_SHAPES:
+            row = {"shape": [M, N, K]}
+            for name in ("A col-major", "A row-major"):
+                a = torch.empty((K, M) if name == "A col-major" else (M, K), device="cuda", dtype=torch.half).uniform_(-1, 1)
+                b = torch.empty(N, K, device="cuda", dtype=torch.half).uniform_(-1, 1)      # column-major B
+                fn = (lambda: torch.matmul(b, a)) if name == "A col-major" else (lambda: torch.matmul(a, b.t()))
+                t0 = time.perf_counter()
+                while time.perf_counter() - t0 < 0.25:
+                    for _ in range(20):
+                        fn()
+                    torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(30):
+                    fn()
+                torch.cuda.synchronize()
+                row[name] = {"us": round((time.perf_counter() - t0) / 30 * 1e6, 1)}
+                del a, b
+            out.append(row)
+        print(json.dumps({"shape_sweep": "torch.matmul Float16 (torch %s)" % torch.__version__, "rows": out}))
+        return
+    from __graft_entry__ import load_package
+    m = load_package()
+    m.init(0)
+    W, G = m.WMMA, m.GEMM
+    names = {v["id"]: v["name"] for v in G.variants()}
+    rng = np.random.default_rng(0)
+
+    def timed(desc, bufs, spin):
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < spin:
+            G.gemm_bench(*bufs, desc, warmup=0, iters=20)
+        return float(np.median(G.gemm_bench(*bufs, desc, warmup=5, iters=30))) * 1e3
+
+    for M, N, K in SWEEP_SHAPES:
+        bufs = (m.DeviceArray(rng.uniform(-1, 1, M * K).astype(np.float16)), m.DeviceArray(rng.uniform(-1, 1, K * N).astype(np.float16)),
+                m.DeviceArray(rng.uniform(-1, 1, M * N).astype(np.float32)), m.DeviceArray.undef(np.float32, M * N))
+        row = {"shape": [M, N, K]}
+        for name, la in (("A col-major", W.ColMajor), ("A row-major", W.RowMajor)):
+            desc = G.make_desc(M, N, K, a_layout=la)
+            plan = G.plan(desc)
+            r = {"us": round(timed(desc, bufs, 0.25), 1),
+                 "launches": ["%s %dx%dx%d" % (names[q["variant"]], q["m"], q["n"], q["k"]) for q in plan]}
+            best = None
+            for v in G.variants():
+                d2 = G.make_desc(M, N, K, a_layout=la, variant=v["id"])
+                if v["fragment_ops"] or not G.variant_supports(d2, v["id"]) or (len(plan) == 1 and plan[0]["variant"] == v["id"]):
+                    continue
+                t = timed(d2, bufs, 0.1)
+                if best is None or t < best[0]:
+                    best = (t, v["name"])
+            if best:
+                r["best_other_single_variant"] = {"us": round(best[0], 1), "variant": best[1]}
+            row[name] = r
+        out.append(row)
+        del bufs
+    print(json.dumps({"shape_sweep": "miw_gemm, Float32 C and D", "library_build_id": m._lib.load().miw_build_id().decode(), "rows": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -128,6 +203,9 @@ def main():
     ap.add_argument("--library-reference", action="store_true",
                     help="instead of this library, time the vendor GEMM (hipBLASLt / rocBLAS through torch.matmul) on "
                          "4096^3 Float16 operands in the four operand layouts and print one line; a comparison aid")
+    ap.add_argument("--shape-sweep", choices=("library", "vendor"),
+                    help="instead of the benchmark, time a list of shapes (sizes tiles divide, ragged and thin ones): "
+                         "'library' this library's own choice of launches beside every single variant, 'vendor' torch.matmul")
     ap.add_argument("--operand-scale", type=float, default=1.0,
                     help="multiply A and B by this before rounding to Float16 (0: all-zero operands, which lift the "
                          "power cap off the matrix cores; a measurement aid, not the benchmark)")
@@ -147,6 +225,9 @@ def main():
 
     if args.library_reference:
         library_reference()
+        return
+    if args.shape_sweep:
+        shape_sweep(args.shape_sweep == "vendor")
         return
     from __graft_entry__ import load_package
     from oracle import oracle as orc
