@@ -468,32 +468,71 @@ __global__ __launch_bounds__(1024) void k_gemm_fragops_ksplit(gemm_params p, int
     fragment<accumulator, 16, 16, 16, float, layout::unspecified> acc[T];
 #pragma unroll
     for (int t = 0; t < T; t++) acc[t] = fill_c<cfg32, float>(0.f);
-    // The K loop, once per combination of operand layouts (they are uniform over the grid): the
-    // loads of a fragment are 8 contiguous bytes per lane where k is contiguous.
-    auto walk = [&]<bool AR, bool BR>(std::bool_constant<AR>, std::bool_constant<BR>) {
+    // The K loop, once per combination of operand layouts (they are uniform over the grid).  With K a
+    // multiple of 32 a step is 32 k-values on v_mfma_f32_16x16x32_f16 (lane (q, r) holds k = 8q .. 8q + 7
+    // of row, or column, r: 16 contiguous bytes per lane where k is contiguous, and the same
+    // accumulator layout); otherwise 16 k-values through load_a / load_b / mma.
+    auto walk = [&]<bool AR, bool BR, bool K32>(std::bool_constant<AR>, std::bool_constant<BR>, std::bool_constant<K32>) {
         constexpr layout la = AR ? layout::row_major : layout::col_major, lb = BR ? layout::row_major : layout::col_major;
-        for (long k0 = 16l * wave; k0 < p.K; k0 += 16l * S) {
-            if (T > 1 && !thin_m) {
-                const auto a = load_a<cfg32, la>(A + tile_offset(la, (int)(tm0 * 16), 0, p.lda) + tile_offset(la, 0, (int)k0, p.lda), p.lda);
+        if constexpr (K32) {
+            const int q = lane >> 4, r = lane & 15;
+            auto wide_a = [&](long tm, long k0) {
+                half8_t v;
 #pragma unroll
-                for (int t = 0; t < T; t++) {
-                    const auto b = load_b<cfg32, lb>(B + tile_offset(lb, (int)k0, 0, p.ldb) + tile_offset(lb, 0, t * 16, p.ldb), p.ldb);
-                    acc[t] = mma<cfg32>(a, b, acc[t]);
+                for (int e = 0; e < 8; e++) v[e] = A[tile_offset(la, (int)(tm * 16) + r, (int)k0 + 8 * q + e, p.lda)];
+                return v;
+            };
+            auto wide_b = [&](long tn, long k0) {
+                half8_t v;
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = B[tile_offset(lb, (int)k0 + 8 * q + e, (int)(tn * 16) + r, p.ldb)];
+                return v;
+            };
+            float4_t sum[T];
+#pragma unroll
+            for (int t = 0; t < T; t++) sum[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+            for (long k0 = 32l * wave; k0 < p.K; k0 += 32l * S) {
+                if (T > 1 && !thin_m) {
+                    const half8_t a = wide_a(tm0, k0);
+#pragma unroll
+                    for (int t = 0; t < T; t++) sum[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, wide_b(t, k0), sum[t], 0, 0, 0);
+                } else {
+                    const half8_t b = wide_b(tn0, k0);
+#pragma unroll
+                    for (int t = 0; t < T; t++) sum[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wide_a(tm0 + t, k0), b, sum[t], 0, 0, 0);
                 }
-            } else {
-                const auto b = load_b<cfg32, lb>(B + tile_offset(lb, (int)k0, 0, p.ldb) + tile_offset(lb, 0, (int)(tn0 * 16), p.ldb), p.ldb);
+            }
 #pragma unroll
-                for (int t = 0; t < T; t++) {
-                    const auto a = load_a<cfg32, la>(A + tile_offset(la, (int)((tm0 + t) * 16), 0, p.lda) + tile_offset(la, 0, (int)k0, p.lda), p.lda);
-                    acc[t] = mma<cfg32>(a, b, acc[t]);
+            for (int t = 0; t < T; t++)
+                for (int i = 0; i < 4; i++) acc[t].x[i] = sum[t][i];
+        } else {
+            for (long k0 = 16l * wave; k0 < p.K; k0 += 16l * S) {
+                if (T > 1 && !thin_m) {
+                    const auto a = load_a<cfg32, la>(A + tile_offset(la, (int)(tm0 * 16), 0, p.lda) + tile_offset(la, 0, (int)k0, p.lda), p.lda);
+#pragma unroll
+                    for (int t = 0; t < T; t++) {
+                        const auto b = load_b<cfg32, lb>(B + tile_offset(lb, (int)k0, 0, p.ldb) + tile_offset(lb, 0, t * 16, p.ldb), p.ldb);
+                        acc[t] = mma<cfg32>(a, b, acc[t]);
+                    }
+                } else {
+                    const auto b = load_b<cfg32, lb>(B + tile_offset(lb, (int)k0, 0, p.ldb) + tile_offset(lb, 0, (int)(tn0 * 16), p.ldb), p.ldb);
+#pragma unroll
+                    for (int t = 0; t < T; t++) {
+                        const auto a = load_a<cfg32, la>(A + tile_offset(la, (int)((tm0 + t) * 16), 0, p.lda) + tile_offset(la, 0, (int)k0, p.lda), p.lda);
+                        acc[t] = mma<cfg32>(a, b, acc[t]);
+                    }
                 }
             }
         }
     };
-    if (p.a_row && p.b_row) walk(std::true_type{}, std::true_type{});
-    else if (p.a_row) walk(std::true_type{}, std::false_type{});
-    else if (p.b_row) walk(std::false_type{}, std::true_type{});
-    else walk(std::false_type{}, std::false_type{});
+    auto walk_k = [&]<bool AR, bool BR>(std::bool_constant<AR> ar, std::bool_constant<BR> br) {
+        if (p.K % 32 == 0) walk(ar, br, std::true_type{});
+        else walk(ar, br, std::false_type{});
+    };
+    if (p.a_row && p.b_row) walk_k(std::true_type{}, std::true_type{});
+    else if (p.a_row) walk_k(std::true_type{}, std::false_type{});
+    else if (p.b_row) walk_k(std::false_type{}, std::true_type{});
+    else walk_k(std::false_type{}, std::false_type{});
     if (wave) {
 #pragma unroll
         for (int t = 0; t < T; t++)
