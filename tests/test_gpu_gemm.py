@@ -513,7 +513,8 @@ def test_thin_problems_share_a_tile_between_wavefronts(gpu, orc, al, bl, cl, dl)
                                        (272, 48, 1024, dict(beta=0.5)), (64, 272, 1040, dict(d_type=orc.F16, c_type=orc.F16)),
                                        # all tiles of the thin dimension in one workgroup (2, 3 and 4 of them)
                                        (32, 1024, 512, dict(beta=-1.0)), (1024, 48, 512, dict(alpha=2.0, batch=2)),
-                                       (64, 1024, 528, dict(d_type=orc.F16, c_type=orc.F16))]):
+                                       (64, 1024, 528, dict(d_type=orc.F16, c_type=orc.F16)),
+                                       (64, 4096, 2064, dict(d_type=orc.F16, c_type=orc.F16))]):   # 16 wavefronts x 4 tiles: 64 KiB of partial sums
         g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl,
                          ldd=(N if dl == orc.ROW else M) + 8, **kw)
         assert [q["variant"] for q in _plan(gpu, orc, g)][-1] == frag
