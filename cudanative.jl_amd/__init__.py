@@ -9,8 +9,9 @@ import ctypes as _ctypes
 
 from . import _lib
 from ._lib import MIWError, DeviceInfo
-from .array import AS, DeviceArray, DevicePtr, CU_NULL, pointer
-from .execution import HostKernel, Module, Stream, cuda, cufunction, cudaconvert, kernel_names, synchronize
+from .array import AS, DeviceArray, DevicePtr, CU_NULL, pointer, mem_info
+from .execution import (HostKernel, Module, Stream, cuda, cufunction, cudaconvert, kernel_names, synchronize,
+                        warpsize, nextwarp, prevwarp)
 from . import wmma as WMMA
 from . import gemm as GEMM
 from . import reflection

@@ -117,6 +117,7 @@ SIGNATURES = {
     "miw_memcpy_d2h": (_i, [_vp, _vp, _sz]),
     "miw_memcpy_d2d": (_i, [_vp, _vp, _sz]),
     "miw_memset": (_i, [_vp, _i, _sz]),
+    "miw_mem_info": (_i, [ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
     "miw_stream_create": (_i, [_vpp]),
     "miw_stream_destroy": (_i, [_vp]),
     "miw_sync": (_i, [_vp]),
@@ -141,10 +142,12 @@ SIGNATURES = {
     "miw_gemm_pick_variant": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
     "miw_gemm_plan": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(GemmPart), _i, ctypes.POINTER(_i)]),
     "miw_gemm_acc_chunk": (_i, [ctypes.POINTER(GemmDesc), ctypes.POINTER(_i)]),
+    "miw_gemm_resolve": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, ctypes.POINTER(_i), ctypes.POINTER(_i)]),
     "miw_gemm_splitk_workspace": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
     "miw_gemm_splitk": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "miw_gemm_splitk_static": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _i, _vp]),
     "miw_gemm_splitk_static_capacity": (_sz, []),
+    "miw_gemm_splitk_static_plan": (_i, [ctypes.POINTER(GemmDesc), _i, ctypes.POINTER(_i), ctypes.POINTER(_sz)]),
     "miw_gemm_bench": (_i, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp, _vp, _i, _i, ctypes.POINTER(_f)]),
     "miw_launch_overhead_probe": (_i, [_i, _i, ctypes.POINTER(_f), ctypes.POINTER(_f)]),
     "miw_mfma_power_probe": (_i, [_i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), _vp]),

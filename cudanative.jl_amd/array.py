@@ -148,5 +148,12 @@ class DeviceArray:
         _lib.check(_lib.load().miw_memset(self.ptr, byte, self.nbytes))
 
 
+def mem_info():
+    """(free, total) bytes of device memory."""
+    f, t = ctypes.c_size_t(), ctypes.c_size_t()
+    _lib.check(_lib.load().miw_mem_info(ctypes.byref(f), ctypes.byref(t)))
+    return f.value, t.value
+
+
 def pointer(a, index=1):
     return a.pointer(index)

@@ -10,7 +10,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmiwmma.so")
-SOURCES = ["gemm_tile_256x256_w2x4.hip", "gemm_tile_256x128.hip", "gemm_tile_256x256_w2x2.hip", "gemm_tile_small.hip", "gemm_tile_pp.hip", "gemm_tile_pp64.hip",
+SOURCES = ["gemm_tile_256x128.hip", "gemm_tile_256x256_w2x2.hip", "gemm_tile_small.hip", "gemm_tile_pp.hip", "gemm_tile_pp64.hip",
            "capi.hip", "frag_kernels.hip", "gemm_kernels.hip"]
 
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
@@ -37,6 +37,23 @@ def source_id():
         with open(f, "rb") as fh:
             h.update(fh.read())
     return h.hexdigest()[:16]
+
+
+def built_id(path=None):
+    """Build id of the library file at `path`, read from the file's bytes (the id follows the marker
+    "miw-build-id:"); None when the file is missing or carries no id.  Loading the library to ask it
+    would pin that binary in the asking process: a later rebuild at the same path would not be seen."""
+    path = path or LIB
+    try:
+        with open(path, "rb") as fh:
+            data = fh.read()
+    except OSError:
+        return None
+    at = data.find(b"miw-build-id:")
+    if at < 0:
+        return None
+    end = data.find(b"\0", at)
+    return data[at + 13:end].decode(errors="replace")
 
 
 def hipcc():

@@ -156,7 +156,7 @@ bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f
     const miw::tiled_variant &v = miw::tiled_variant_at(i);
     // In canonical terms bm tiles the contiguous dimension of D.
     const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
-    if (I < v.bm || J < v.bn || p.K % v.bk) return false;
+    if (I < v.bm || J < v.bn || p.K < v.bk) return false;  // (K is a multiple of 16: a last slot that 64 does not divide is shifted back and masked)
     if ((I % v.bm || J % v.bn) && in_place) return false;
     if (!miw::tiled_supports_layout(i, p) || !miw::tiled_grid_fits(i, p)) return false;
     if (!aligned16(p.A) || !aligned16(p.B) || !aligned16(p.D) || (p.use_c && !aligned16(p.C))) return false;
@@ -182,6 +182,56 @@ std::mutex g_module_mu;
 std::unordered_map<void *, void *> g_module_kernels;
 std::unordered_map<void *, int> g_modules;
 
+// Do the headers of a code object image stay inside its buffer?  ELF64: the section header table and
+// every section with file contents; clang offload bundle: every entry's offset + size, and each
+// entry that is an ELF by the same rule.
+bool elf_fits(const unsigned char *img, size_t bytes)
+{
+    if (bytes < 64 || memcmp(img, "\177ELF", 4) != 0 || img[4] != 2 /* ELFCLASS64 */) return false;
+    uint64_t shoff;
+    uint16_t shentsize, shnum;
+    memcpy(&shoff, img + 0x28, 8);
+    memcpy(&shentsize, img + 0x3a, 2);
+    memcpy(&shnum, img + 0x3c, 2);
+    if (shnum == 0) return true;
+    if (shentsize < 64 || shoff > bytes || (uint64_t)shnum * shentsize > bytes - shoff) return false;
+    for (unsigned i = 0; i < shnum; i++) {
+        const unsigned char *sh = img + shoff + (uint64_t)i * shentsize;
+        uint32_t type;
+        uint64_t off, size;
+        memcpy(&type, sh + 4, 4);
+        memcpy(&off, sh + 0x18, 8);
+        memcpy(&size, sh + 0x20, 8);
+        if (type == 8 /* SHT_NOBITS */) continue;
+        if (off > bytes || size > bytes - off) return false;
+    }
+    return true;
+}
+
+bool image_fits(const void *image, size_t bytes)
+{
+    const unsigned char *img = (const unsigned char *)image;
+    if (bytes >= 4 && memcmp(img, "\177ELF", 4) == 0) return elf_fits(img, bytes);
+    // __CLANG_OFFLOAD_BUNDLE__ (24 bytes), u64 entry count, then per entry: u64 offset, u64 size, u64 id length, id
+    if (bytes < 32) return false;
+    uint64_t n;
+    memcpy(&n, img + 24, 8);
+    size_t at = 32;
+    for (uint64_t i = 0; i < n; i++) {
+        if (at > bytes || bytes - at < 24) return false;
+        uint64_t off, size, idlen;
+        memcpy(&off, img + at, 8);
+        memcpy(&size, img + at + 8, 8);
+        memcpy(&idlen, img + at + 16, 8);
+        at += 24;
+        if (idlen > bytes - at) return false;
+        at += idlen;
+        if (off > bytes || size > bytes - off) return false;
+        if (size >= 4 && memcmp(img + off, "\177ELF", 4) == 0 && !elf_fits(img + off, size)) return false;
+    }
+    return true;
+}
+
 bool is_module_kernel(void *kernel)
 {
     std::lock_guard<std::mutex> lock(g_module_mu);
@@ -203,7 +253,7 @@ double estimate_us(int i, const miw::gemm_params &p, int c_type, int d_type)
     const long rounds = (per_cu + v.occupancy - 1) / v.occupancy;
     const double per_pair = std::max((double)v.us_pair_alone, (double)per_cu * v.us_pair_queued);
     const double cd_bytes = (double)I * (double)J * (double)p.batch * (double)(dtype_size(d_type) + (p.use_c ? dtype_size(c_type) : 0));
-    return 4.5 * (double)rounds + cd_bytes / 5.5e6 + (double)(p.K / v.bk) * per_pair;
+    return 4.5 * (double)rounds + cd_bytes / 5.5e6 + (double)((p.K + v.bk - 1) / v.bk) * per_pair;
 }
 
 // Tiled variants from large tiles to small, of two kernels for one tile the ping-pong form first.
@@ -277,8 +327,6 @@ int launch_gemm(int variant, const miw::gemm_params &p, int c_type, int d_type, 
 // and D share memory: then only whole tiles).  Beyond that a problem may be cut into parts, each
 // a GEMM of its own on a block of D (same leading dimensions and batch strides, offset
 // pointers), launched one after the other on the caller's stream:
-//   * K = 64 q + r (Float32 D): the first 64 q k-values by the tiled kernels, the last r by the
-//     fragment-op kernel with D as its C operand (one more Float32 rounding per element);
 //   * a body of whole large tiles plus a bottom strip and a right strip, each planned again
 //     (4160 rows: sixteen rows of 256 x 256 tiles and a strip of 64 x 64 tiles instead of
 //     seventeen rows of large tiles, i.e. two rounds over the CUs).
@@ -337,20 +385,7 @@ struct gemm_planner {
             if (us < 0.97 * best_us) { best_us = us; best.swap(cand); }
         };
         if (depth < 4) {
-            const long k64 = p.K / 64 * 64;
-            if (k64 != p.K && k64 > 0 && d_type == MIW_F32) {
-                miw::gemm_params body = p, tail = p;
-                body.K = k64;
-                tail.K = p.K - k64;
-                tail.A = p.A + k64 * (p.a_row ? 1 : p.lda);
-                tail.B = p.B + k64 * (p.b_row ? p.ldb : 1);
-                tail.C = p.D; tail.use_c = 1; tail.beta = 1.0f;
-                tail.c_row = p.d_row; tail.ldc = p.ldd; tail.sc = p.sd;
-                std::vector<gemm_part> cand;
-                double us = plan(body, c_type, m0, n0, k0, depth + 1, &cand);
-                us += single(tail, d_type, m0, n0, k0 + k64, &cand);
-                offer(cand, us);
-            } else if (k64 == p.K) {
+            if (p.K >= 64) {
                 // whole large tiles, then what they leave at the bottom and on the right; a strip
                 // is widened backwards to 64 rows (columns), over the body, where that is allowed
                 for (int i : variant_order()) {
@@ -448,7 +483,10 @@ const char *miw_last_error(void) { return g_err; }
 #ifndef MIW_BUILD_ID
 #define MIW_BUILD_ID "unknown"
 #endif
-const char *miw_build_id(void) { return MIW_BUILD_ID; }
+// The id follows a marker in the binary, so that a build script or test harness can read it from the
+// file without loading the library into its own process.
+static const char g_build_id[] = "miw-build-id:" MIW_BUILD_ID;
+const char *miw_build_id(void) { return g_build_id + 13; }
 
 int miw_init(int device)
 {
@@ -802,6 +840,19 @@ int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk)
     return 0;
 }
 
+int miw_gemm_resolve(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, const void *D, int *variant, int *acc_chunk)
+{
+    miw::gemm_params p;
+    bool f16acc;
+    if (int rc = resolve_gemm(desc, A, B, C, const_cast<void *>(D), &p, &f16acc)) return rc;
+    std::vector<gemm_part> parts;
+    if (int rc = plan_gemm(desc, p, f16acc, c_shares_d(desc, p), &parts)) return rc;
+    const int v = parts.empty() ? 0 : parts[0].variant;
+    if (variant) *variant = v;
+    if (acc_chunk) *acc_chunk = !f16acc ? 0 : v == miw::tiled_variant_count() + 1 ? 16 : miw::tiled_f16acc_chunk();
+    return 0;
+}
+
 int miw_gemm(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream)
 {
     miw::gemm_params p;
@@ -870,7 +921,8 @@ miw::gemm_params splitk_slices(const miw::gemm_params &p, int splits, void *ws)
     return q;
 }
 
-int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void *C, void *D, int splits, splitk_plan *out)
+int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void *C, void *D, int splits, splitk_plan *out,
+                size_t workspace_cap = SIZE_MAX)
 {
     bool f16acc;
     miw::gemm_params p;
@@ -911,6 +963,8 @@ int plan_splitk(const miw_gemm_desc *d, const void *A, const void *B, const void
         double best_us = 0.0;
         for (int s = 1; s <= 64 && (s == 1 || p.K / s >= 128); s++) {
             int v;
+            // a caller with a bounded workspace is offered only the counts that fit in it
+            if (s > 1 && (size_t)s * (size_t)p.M * (size_t)p.N * sizeof(float) > workspace_cap) break;
             if (!try_splits(s, &v, &us)) continue;
             if (splits == 0 || us < 0.97 * best_us) { splits = s; variant = v; best_us = us; }
         }
@@ -980,7 +1034,7 @@ int miw_gemm_splitk_static(const miw_gemm_desc *desc, const void *A, const void 
                            void *stream)
 {
     splitk_plan plan;
-    if (int rc = plan_splitk(desc, A, B, C, D, splits, &plan)) return rc;
+    if (int rc = plan_splitk(desc, A, B, C, D, splits, &plan, SPLITK_STATIC_BYTES)) return rc;
     if (plan.bytes > SPLITK_STATIC_BYTES)
         return fail(MIW_ERR_UNSUPPORTED,
                     "gemm_splitk_static: %d slices of %lld x %lld Float32 need %zu bytes, the static workspace holds %zu; "
@@ -993,6 +1047,29 @@ int miw_gemm_splitk_static(const miw_gemm_desc *desc, const void *A, const void 
 }
 
 size_t miw_gemm_splitk_static_capacity(void) { return SPLITK_STATIC_BYTES; }
+
+int miw_gemm_splitk_static_plan(const miw_gemm_desc *desc, int splits, int *splits_out, size_t *bytes)
+{
+    if (!bytes) return fail(MIW_ERR_NULL_POINTER, "gemm_splitk_static_plan: null output");
+    char *const base = (char *)(uintptr_t)0x100000000ull;
+    splitk_plan plan;
+    if (int rc = plan_splitk(desc, base, base + (1ull << 40), base + (2ull << 40), base + (3ull << 40), splits, &plan, SPLITK_STATIC_BYTES))
+        return rc;
+    if (plan.bytes > SPLITK_STATIC_BYTES)
+        return fail(MIW_ERR_UNSUPPORTED, "gemm_splitk_static: %d slices need %zu bytes, the static workspace holds %zu", plan.splits,
+                    plan.bytes, SPLITK_STATIC_BYTES);
+    if (splits_out) *splits_out = plan.splits;
+    *bytes = plan.bytes;
+    return 0;
+}
+
+int miw_mem_info(size_t *free_bytes, size_t *total_bytes)
+{
+    if (!free_bytes || !total_bytes) return fail(MIW_ERR_NULL_POINTER, "mem_info: null output");
+    REQUIRE_INIT("mem_info");
+    HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));
+    return 0;
+}
 
 int miw_gemm_bench(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, void *stream,
                    int warmup, int iters, float *ms_each)
@@ -1220,6 +1297,9 @@ int miw_module_load(const void *image, size_t bytes, void **module)
     const bool bundle = bytes >= sizeof(bundle_magic) - 1 && memcmp(image, bundle_magic, sizeof(bundle_magic) - 1) == 0;
     if (!elf && !bundle)
         return fail(MIW_ERR_INVALID_VALUE, "module_load: %zu bytes that are neither an ELF code object nor an offload bundle", bytes);
+    // hipModuleLoadData takes no size: it reads as far as the image's own headers say.  Check that they stay inside the buffer.
+    if (!image_fits(image, bytes))
+        return fail(MIW_ERR_INVALID_VALUE, "module_load: the image's headers describe more than the %zu bytes given (truncated file?)", bytes);
     REQUIRE_INIT("module_load");
     hipModule_t m = nullptr;
     HIP_TRY(hipModuleLoadData(&m, image));

@@ -334,7 +334,11 @@ __global__ __launch_bounds__(256) void k_gemm_shortk(shortk_params p)
     DT *D = (DT *)p.D + bt * p.sd;
 
     // Both operand blocks (64 rows of X, 64 columns of Y, all of K) go to LDS with k contiguous, in
-    // 16-byte pieces along whichever dimension is contiguous in memory; rows past the edge repeat the last one.
+    // 16-byte pieces along whichever dimension is contiguous in memory.  A block that reaches past the
+    // edge (extents are multiples of 16, blocks of 64) has rows nobody stores: with k contiguous they
+    // repeat the last row; otherwise the last 8-row piece is shifted back to end at the edge and the
+    // rows beyond it keep whatever LDS held.  Either way they only feed output rows or columns that the
+    // epilogue masks out.
     const int K = (int)p.K, kc = K / 8;
     auto stage_operand = [&](half_t *dst, const half_t *src, long ld, bool k_contiguous, long first, long extent) {
         if (k_contiguous) {

@@ -14,7 +14,6 @@ namespace miw {
 static const tiled_variant g_variants[] = {
     // name                    bm   bn  bk     wm wn slots lds, kind (32-k ping-pong: ring depth of a K-major operand, largest ring),
     //                                                          workgroups per CU, us per 64 k alone, us per 64 k in a queue
-    {"tile256x256_w2x4", 256, 256, KGRAN, 2, 4, 2, 2 * (256 + 256) * KGRAN * 2, 0, 1, 1.37f, 1.37f},
     {"tile256x256_w2x2", 256, 256, KGRAN, 2, 2, 2, 2 * (256 + 256) * KGRAN * 2, 0, 1, 1.55f, 1.55f},
     {"tile256x128_w4x2", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 0, 1, 0.80f, 0.80f},
     {"tile128x256_w2x4", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 0, 1, 0.80f, 0.80f},
@@ -40,7 +39,6 @@ bool tiled_supports_f16acc(int i)
 }
 
 // One lookup per tile family, each defined in its own translation unit.
-const void *tiled_kernel_256x256_w2x4(bool xk, bool yk, int c_type, int d_type, bool f16acc);
 const void *tiled_kernel_256x256_w2x2(bool xk, bool yk, int c_type, int d_type, bool f16acc);
 const void *tiled_kernel_256x128_w4x2(bool xk, bool yk, int c_type, int d_type, bool f16acc);
 const void *tiled_kernel_128x256_w2x4(bool xk, bool yk, int c_type, int d_type, bool f16acc);
@@ -56,18 +54,17 @@ const void *pp64_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type
 // Tile shape in canonical (I, J) terms: bm applies to I, bn to J.
 static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, bool f16acc)
 {
-    switch (i) {
-        case 0: return tiled_kernel_256x256_w2x4(xk, yk, c_type, d_type, f16acc);
-        case 1: return tiled_kernel_256x256_w2x2(xk, yk, c_type, d_type, f16acc);
-        case 2: return tiled_kernel_256x128_w4x2(xk, yk, c_type, d_type, f16acc);
-        case 3: return tiled_kernel_128x256_w2x4(xk, yk, c_type, d_type, f16acc);
-        case 4: return tiled_kernel_128x128_w2x4_s4(xk, yk, c_type, d_type, f16acc);
-        case 5: return tiled_kernel_128x128_w2x2_s4(xk, yk, c_type, d_type, f16acc);
-        case 6: return tiled_kernel_128x128_w2x2(xk, yk, c_type, d_type, f16acc);
-        case 7: return tiled_kernel_64x64_w2x2(xk, yk, c_type, d_type, f16acc);
-        case 8: return f16acc ? nullptr : pp_kernel(256, 256, xk, yk, c_type, d_type);
-        case 9: case 10: case 11: return pp64_kernel(g_variants[i].bm, g_variants[i].bn, xk, yk, c_type, d_type, f16acc);
-    }
+    const tiled_variant &v = g_variants[i];
+    if (v.kind == KIND_PINGPONG32) return f16acc ? nullptr : pp_kernel(v.bm, v.bn, xk, yk, c_type, d_type);
+    if (v.kind == KIND_PINGPONG64) return pp64_kernel(v.bm, v.bn, xk, yk, c_type, d_type, f16acc);
+    const int waves = v.wm * v.wn;
+    if (v.bm == 256 && v.bn == 256 && waves == 4) return tiled_kernel_256x256_w2x2(xk, yk, c_type, d_type, f16acc);
+    if (v.bm == 256 && v.bn == 128) return tiled_kernel_256x128_w4x2(xk, yk, c_type, d_type, f16acc);
+    if (v.bm == 128 && v.bn == 256) return tiled_kernel_128x256_w2x4(xk, yk, c_type, d_type, f16acc);
+    if (v.bm == 128 && v.bn == 128 && waves == 8) return tiled_kernel_128x128_w2x4_s4(xk, yk, c_type, d_type, f16acc);
+    if (v.bm == 128 && v.bn == 128 && v.stages == 4) return tiled_kernel_128x128_w2x2_s4(xk, yk, c_type, d_type, f16acc);
+    if (v.bm == 128 && v.bn == 128) return tiled_kernel_128x128_w2x2(xk, yk, c_type, d_type, f16acc);
+    if (v.bm == 64 && v.bn == 64) return tiled_kernel_64x64_w2x2(xk, yk, c_type, d_type, f16acc);
     return nullptr;
 }
 
@@ -95,7 +92,7 @@ bool tiled_supports_layout(int i, const gemm_params &g)
     if (g_variants[i].kind != KIND_PINGPONG32) return true;
     bool xk, yk;
     canonical_layout(g, &xk, &yk);
-    return pp_kernel(g_variants[i].bm, g_variants[i].bn, xk, yk, 1, 1) != nullptr;  // two K-major 256-row rings do not fit in LDS
+    return pp_kernel(g_variants[i].bm, g_variants[i].bn, xk, yk, 1, 1) != nullptr;  // (every layout has a ring that fits in LDS at 256 x 256)
 }
 
 // hipFuncAttributeMaxDynamicSharedMemorySize is a property of the kernel, not of the launch: set once.

@@ -24,6 +24,15 @@
 // a load has two full clusters of both groups (about 2000 cycles) to land
 // before anyone waits for it, and the barriers between that wait and the first
 // read publish it to the other wavefronts.
+//   Two K-major operands: three slots each would be 192 KiB.  X keeps three, Y
+//       gets two (160 KiB).  A slot of Y is free once both groups have read its
+//       second k-step, which is when group 0 starts the memory cluster after
+//       that; so the first cluster of pair p+1 requests all of Y's pair p+2
+//       into the slot of pair p, and the wait at the end of the second cluster
+//       of pair p+1 must cover it: that cluster leaves only its own loads in
+//       flight, and those are X's (all of X's pair p+3, into the slot of pair
+//       p).  Y's loads have one compute and one memory cluster to land, X's two
+//       of each as before.
 #pragma once
 #include "gemm_tiled.hpp"
 
@@ -35,6 +44,7 @@ namespace miw {
 #ifndef MIW_PP_ABLATE
 #define MIW_PP_ABLATE 0
 #endif
+
 
 // Second measurement switch (off in every shipped build; gemm_kernels.hip must be compiled with it
 // too): with MIW_PP_TS the ping-pong kernels record, per wavefront, the shader clock at kernel
@@ -52,23 +62,28 @@ namespace miw {
 constexpr int PP_KMAJOR_SLOTS = 3;
 constexpr int PP_IMAJOR_ENTRIES = 4;
 
-constexpr int pp_operand_bytes(int rows, bool kmajor)
+// Slots of a K-major Y: two when X is K-major as well (see above), else three.
+constexpr int pp_y_slots(bool xk) { return xk ? 2 : PP_KMAJOR_SLOTS; }
+constexpr int pp_operand_bytes(int rows, bool kmajor, int kslots)
 {
-    return kmajor ? PP_KMAJOR_SLOTS * rows * KGRAN * 2 : PP_IMAJOR_ENTRIES * rows * BKS * 2;
+    return kmajor ? kslots * rows * KGRAN * 2 : PP_IMAJOR_ENTRIES * rows * BKS * 2;
 }
-constexpr int pp_lds_bytes(int bi, int bj, bool xk, bool yk) { return pp_operand_bytes(bi, xk) + pp_operand_bytes(bj, yk); }
+constexpr int pp_lds_bytes(int bi, int bj, bool xk, bool yk)
+{
+    return pp_operand_bytes(bi, xk, PP_KMAJOR_SLOTS) + pp_operand_bytes(bj, yk, pp_y_slots(xk));
+}
 constexpr bool pp_fits(int bi, int bj, bool xk, bool yk) { return pp_lds_bytes(bi, bj, xk, yk) <= 160 * 1024; }
 
 // One operand of the ping-pong kernel: its ring in LDS, the loads that fill it
 // and the fragment reads.  R rows (or columns) of the tile, NT threads.
-template <int R, bool KMAJOR, int NT>
+template <int R, bool KMAJOR, int NT, int KSLOTS = PP_KMAJOR_SLOTS>
 struct pp_operand {
     // loads per thread: per 64-k slot (K-major) or per 32-k entry (I-major)
     static constexpr int NL = KMAJOR ? R * KGRAN / 8 / NT : R * BKS / 8 / NT;
-    // loads per thread and memory cluster
+    // loads per thread and memory cluster (a K-major operand: half a slot, unless both operands are K-major)
     static constexpr int PER_CLUSTER = KMAJOR ? NL / 2 : NL;
     static constexpr int UNIT_BYTES = KMAJOR ? R * KGRAN * 2 : R * BKS * 2;
-    static constexpr int UNITS = KMAJOR ? PP_KMAJOR_SLOTS : PP_IMAJOR_ENTRIES;
+    static constexpr int UNITS = KMAJOR ? KSLOTS : PP_IMAJOR_ENTRIES;
     static constexpr int BYTES = UNITS * UNIT_BYTES;
     static_assert(NL >= 1 && (!KMAJOR || NL % 2 == 0), "operand must divide over the workgroup");
     static_assert(NT == 512, "lane offsets below assume 512 threads");
@@ -90,8 +105,6 @@ struct pp_operand {
         if constexpr (KMAJOR) return (long)i * (NT / 8) * ld;
         else return (long)i * (NT / 256) * 64;
     }
-    // Elements between consecutive units in global memory.
-    __device__ static inline long unit_step(long ld) { return KMAJOR ? (long)KGRAN : (long)BKS * ld; }
 
     // Fragment reads.  K-major: the reader of gemm_tiled.hpp on a 64-k slot.
     // I-major: the same transpose reads on an entry of 32 k-rows (i-blocks of
@@ -137,10 +150,12 @@ void k_gemm_pp(tiled_params p)
     static_assert(NT == 512, "two wavefronts per SIMD");
     constexpr int WTI = BI / WI, WTJ = BJ / WJ;
     constexpr int TI = WTI / 16, TJ = WTJ / 16;
+    constexpr bool KK = XK && YK;  // two K-major operands: Y has two slots, clusters alternate between Y's loads and X's
     using xop = pp_operand<BI, XK, NT>;
-    using yop = pp_operand<BJ, YK, NT>;
+    using yop = pp_operand<BJ, YK, NT, pp_y_slots(XK)>;
     constexpr int XB = xop::BYTES;
     constexpr int ND = xop::PER_CLUSTER + yop::PER_CLUSTER;  // loads per thread and memory cluster
+    static_assert(!KK || (xop::NL == ND && yop::NL == ND), "alternating clusters carry equal loads");
     static_assert(pp_fits(BI, BJ, XK, YK), "ring does not fit in LDS");
 
 #ifdef MIW_PP_TS
@@ -202,8 +217,10 @@ void k_gemm_pp(tiled_params p)
 #pragma unroll
         for (int b = 0; b < TJ; b++) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const int NS = p.K / BKS;    // k-steps
-    const int NP = p.K / KGRAN;  // pairs of k-steps
+    const int NP = (p.K + KGRAN - 1) / KGRAN;  // pairs of k-steps
+    const int NS = 2 * NP;                     // k-steps
+    // K tail: the last pair starts at K - 64; tail_skip of its k-values repeat the pair before
+    const int tail_skip = NP * KGRAN - p.K;
     const unsigned lds0 = (unsigned)(uintptr_t)lds;
     const unsigned wave_dst = lds0 + (unsigned)wave * 1024u;
 
@@ -211,7 +228,7 @@ void k_gemm_pp(tiled_params p)
     // pair + UNIT_BYTES, pair toggling between 0 and 2 UNIT_BYTES.  K-major operand: `pair` is the
     // slot of the current pair and `prev` the slot of the pair before it, which is the one being
     // refilled (with pair pr + 2).
-    unsigned xpair = 0, xprev = 2 * xop::UNIT_BYTES, ypair = 0, yprev = 2 * yop::UNIT_BYTES;
+    unsigned xpair = 0, xprev = 2 * xop::UNIT_BYTES, ypair = 0, yprev = (yop::UNITS - 1) * yop::UNIT_BYTES;
     int xnext = 0, ynext = 0;  // next unit to request (step index for I-major, pair index for K-major)
     // Lane offsets of the loads of one unit: K-major loads differ by whole rows (a per-load lane
     // offset keeps one uniform base address), I-major loads by 256 bytes (the instruction's offset field).
@@ -230,17 +247,28 @@ void k_gemm_pp(tiled_params p)
         else lds_dma16_at<XB + I * NT * 16, I * 256>(Y, yvo[0], wave_dst + unit);
     };
     // Past the end of K the last unit is requested again, into a unit nobody reads any more.
+    // k-values from one unit to the next; the first unit of the last pair (pair NP - 1, or entry NS - 2)
+    // lies tail_skip short of where it would follow on (a step back for an entry of 32 when 48 repeat).
     auto x_advance = [&]() {
         xnext++;
-        X += xnext < (XK ? NP : NS) ? xop::unit_step(p.ldx) : 0;
+        constexpr int UK = XK ? KGRAN : BKS;
+        const int kstep = xnext == (XK ? NP - 1 : NS - 2) ? UK - tail_skip : xnext < (XK ? NP : NS) ? UK : 0;
+        X += XK ? (long)kstep : (long)kstep * p.ldx;
     };
     auto y_advance = [&]() {
         ynext++;
-        Y += ynext < (YK ? NP : NS) ? yop::unit_step(p.ldy) : 0;
+        constexpr int UK = YK ? KGRAN : BKS;
+        const int kstep = ynext == (YK ? NP - 1 : NS - 2) ? UK - tail_skip : ynext < (YK ? NP : NS) ? UK : 0;
+        Y += YK ? (long)kstep : (long)kstep * p.ldy;
     };
     // Request number N (0 .. ND-1) of the memory cluster of k-step 2 pr + H: the X loads, then the Y loads.
     auto cluster_request = [&]<int H, int N>(std::integral_constant<int, H>, std::integral_constant<int, N>) {
-        if constexpr (N < xop::PER_CLUSTER) {
+        if constexpr (KK) {
+            // first cluster of a pair: all of Y's pair after next, into the slot of the pair before
+            // (read to the end one barrier ago); second cluster: all of X's, likewise
+            if constexpr (H == 0) y_load(yprev, std::integral_constant<int, N>{});
+            else x_load(xprev, std::integral_constant<int, N>{});
+        } else if constexpr (N < xop::PER_CLUSTER) {
             if constexpr (XK) x_load(xprev, std::integral_constant<int, H * xop::NL / 2 + N>{});
             else x_load(H == 0 ? (xpair ^ (2u * xop::UNIT_BYTES)) + xop::UNIT_BYTES : xpair, std::integral_constant<int, N>{});
         } else {
@@ -251,7 +279,7 @@ void k_gemm_pp(tiled_params p)
     };
     auto cluster_advance = [&]<int H>(std::integral_constant<int, H>) {
         if constexpr (!XK || H == 1) x_advance();
-        if constexpr (!YK || H == 1) y_advance();
+        if constexpr (!YK || H == (KK ? 0 : 1)) y_advance();
     };
     auto pair_advance = [&]() {
         if constexpr (XK) {
@@ -268,23 +296,39 @@ void k_gemm_pp(tiled_params p)
         }
     };
 
-    // Prologue: K-major operands request pairs 0 and 1, I-major operands steps 0, 1 and 2; everything
-    // lands and is published before the loop starts.
-#pragma unroll
-    for (int u = 0; u < (XK ? 2 : 3); u++) {
-        [&]<int... I>(std::integer_sequence<int, I...>) {
-            (x_load((unsigned)(u * xop::UNIT_BYTES), std::integral_constant<int, I>{}), ...);
-        }(std::make_integer_sequence<int, xop::NL>{});
-        x_advance();
-    }
-#pragma unroll
-    for (int u = 0; u < (YK ? 2 : 3); u++) {
-        [&]<int... I>(std::integer_sequence<int, I...>) {
-            (y_load((unsigned)(u * yop::UNIT_BYTES), std::integral_constant<int, I>{}), ...);
-        }(std::make_integer_sequence<int, yop::NL>{});
-        y_advance();
-    }
-    wait_loads_and_barrier<0>();
+    // Prologue: K-major operands request pairs 0 and 1, I-major operands steps 0, 1 and 2, in the order
+    // in which the loop needs them: what step 0 reads (unit 0 of each operand), then step 1 (entry 1 of
+    // an I-major operand), then step 2 (entry 2, pair 1).  The loop starts as soon as the units of step
+    // 0 have landed; the rest arrives under the first clusters.  The loop's own wait covers it: at the
+    // end of memory cluster t it leaves 2 ND loads in flight, and the units of step 2 are at least ND
+    // loads, so after cluster 0 the units of step 1 have landed and after cluster 1 those of step 2.
+    auto prologue_unit = [&]<int U>(std::integral_constant<int, U>, bool is_x) {
+        if (is_x) {
+            [&]<int... I>(std::integer_sequence<int, I...>) {
+                (x_load((unsigned)(U * xop::UNIT_BYTES), std::integral_constant<int, I>{}), ...);
+            }(std::make_integer_sequence<int, xop::NL>{});
+            x_advance();
+        } else {
+            [&]<int... I>(std::integer_sequence<int, I...>) {
+                (y_load((unsigned)(U * yop::UNIT_BYTES), std::integral_constant<int, I>{}), ...);
+            }(std::make_integer_sequence<int, yop::NL>{});
+            y_advance();
+        }
+    };
+    constexpr std::integral_constant<int, 0> unit0{};
+    constexpr std::integral_constant<int, 1> unit1{};
+    constexpr std::integral_constant<int, 2> unit2{};
+    prologue_unit(unit0, true);
+    prologue_unit(unit0, false);
+    if constexpr (!XK) prologue_unit(unit1, true);
+    if constexpr (!YK) prologue_unit(unit1, false);
+    if constexpr (XK) prologue_unit(unit1, true);
+    else prologue_unit(unit2, true);
+    if constexpr (!YK) prologue_unit(unit2, false);
+    else if constexpr (!KK) prologue_unit(unit1, false);  // (two K-major operands: cluster 0 requests Y's pair 1)
+    constexpr int PROLOGUE_LOADS = (XK ? 2 : 3) * xop::NL + (KK ? 1 : YK ? 2 : 3) * yop::NL;
+    static_assert(xop::NL + yop::NL >= ND, "the units of step 2 must cover one cluster's requests");
+    wait_loads_and_barrier<PROLOGUE_LOADS - xop::NL - yop::NL>();
 
     half8_t fx[TI], fy[TJ];
     if constexpr (MIW_PP_ABLATE & 2) {
@@ -302,7 +346,8 @@ void k_gemm_pp(tiled_params p)
                                           std::integral_constant<int, U>) {
         [&]<int... N>(std::integer_sequence<int, N...>) {
             (([&] {
-                 if constexpr (N * NFRAG / ND == U && !(MIW_PP_ABLATE & 1)) {
+                 // (Y's loads of a two-K-major kernel have the least time to land: they go out first)
+                 if constexpr ((KK && H == 0 ? N : N * NFRAG / ND) == U && !(MIW_PP_ABLATE & 1)) {
                      cluster_request(h, std::integral_constant<int, N>{});
                      __builtin_amdgcn_sched_barrier(0);
                  }
@@ -379,32 +424,61 @@ void k_gemm_pp(tiled_params p)
         }
     };
     // One k-step: memory cluster, barrier, compute cluster, barrier.  FS >= 0: fold step FS.
+    // Zeroes the repeated k-values in the fragments of step H of the shifted last pair.
+    auto mask_tail = [&]<int H>(std::integral_constant<int, H>) {
+        const unsigned keep = tail_keep<H>(tail_skip);
+#pragma unroll
+        for (int a = 0; a < TI; a++) tail_apply(fx[a], keep);
+#pragma unroll
+        for (int b = 0; b < TJ; b++) tail_apply(fy[b], keep);
+    };
+    // FS >= 0: fold step FS (always folds).  FS == -1: a step that does not fold.  FS == -2: a step of
+    // the last pair: its fragments are masked, and it is fold step NFOLD - 2 + H when the launch folds C,
+    // which is decided here at run time, so that the last pair is one piece of code for both cases (two
+    // alternative pieces that each update all accumulators cost spills where they join).
+    auto fold_wait = [&]<int H, int FS>(std::integral_constant<int, H>, std::integral_constant<int, FS>) {
+        // fold step FS issues ND + CPT loads; steps before the first fold step issue ND
+        constexpr int YOUNGER = (KK && H == 1 ? ND : 2 * ND) + (FS >= 1 ? 2 : 1) * CPT;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt((YOUNGER & 15) | (7 << 4) | (0 << 8) | ((YOUNGER >> 4) << 14));
+        asm volatile("" ::: "memory");
+    };
     auto step = [&]<int H, int FS>(std::integral_constant<int, H> h, std::integral_constant<int, FS>) {
         memory_cluster(h);
         if constexpr (FS >= 0) {
             fold_request(std::integral_constant<int, FS>{});
             __builtin_amdgcn_sched_barrier(0);
-            // fold step FS issues ND + CPT loads; steps before the first fold step issue ND
-            constexpr int YOUNGER = 2 * ND + (FS >= 1 ? 2 : 1) * CPT;
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_waitcnt((YOUNGER & 15) | (7 << 4) | (0 << 8) | ((YOUNGER >> 4) << 14));
-            asm volatile("" ::: "memory");
+            fold_wait(h, std::integral_constant<int, FS>{});
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (FS >= 2) fold_add(std::integral_constant<int, FS - 2>{});
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+        } else if constexpr (FS == -2 && CAN_FOLD) {
+            constexpr int LFS = NFOLD - 2 + H;
+            if (fold_c) {
+                fold_request(std::integral_constant<int, LFS>{});
+                fold_wait(h, std::integral_constant<int, LFS>{});
+                fold_add(std::integral_constant<int, LFS - 2>{});
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            } else {
+                wait_loads_and_barrier<(KK && H == 1 ? ND : 2 * ND)>();
+            }
         } else {
-            wait_loads_and_barrier<2 * ND>();
+            wait_loads_and_barrier<(KK && H == 1 ? ND : 2 * ND)>();
         }
+        if constexpr (FS == -2) mask_tail(h);
         compute_cluster();
         __builtin_amdgcn_s_barrier();
     };
     constexpr std::integral_constant<int, -1> no_fold{};
+    constexpr std::integral_constant<int, -2> last_pair{};
 
     MIW_PP_STAMP(1)
     if (late_group) __builtin_amdgcn_s_barrier();
-    const int NPM = fold_c ? NP - NFOLD / 2 : NP;
+    // the loop runs the pairs that neither fold nor are the last one
+    const int NPM = fold_c ? NP - NFOLD / 2 : NP - 1;
     for (int pr = 0; pr < NPM; pr++) {
 #ifdef MIW_PP_TS
         if (pr == NPM / 2) MIW_PP_STAMP(2)
@@ -420,9 +494,11 @@ void k_gemm_pp(tiled_params p)
                 ((step(std::integral_constant<int, 0>{}, std::integral_constant<int, 2 * G>{}),
                   step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2 * G + 1>{})),
                  ...);
-            }(std::make_integer_sequence<int, NFOLD / 2>{});
+            }(std::make_integer_sequence<int, NFOLD / 2 - 1>{});
         }
     }
+    step(std::integral_constant<int, 0>{}, last_pair);
+    step(std::integral_constant<int, 1>{}, last_pair);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may outlive the workgroup's LDS
     if constexpr (CAN_FOLD) {
         if (fold_c) {
@@ -494,11 +570,12 @@ void k_gemm_pp(tiled_params p)
 // layouts, loaders and fragment readers of gemm_tiled.hpp.
 //
 // fp16 accumulation rounds once per slot (64 k-values), two MFMAs after a tile's last MFMA of the pair,
-// inside the compute cluster; with alpha == 1 the MFMAs accumulate onto the rounded sum in place,
-// otherwise the running sum is kept beside accumulators that restart from zero in every slot:
-// run = half(run + alpha * slot sum) (the memory
-// cluster is the longer of the two at these tiles: it takes about 530 cycles whatever it holds).  The running sum starts as half(beta * C): C is requested before anything else and
-// converted once the prologue's loads have landed.
+// inside the compute cluster: at these tiles the memory cluster is the longer of the two (it is bound
+// by the LDS: measured, the same conversions placed between the fragment reads of the next memory
+// cluster cost 15 to 25 % of the launch).  With alpha == 1 the accumulators start as half(beta * C) and
+// the MFMAs accumulate onto the rounded sum in place, otherwise the running sum is kept beside
+// accumulators that restart from zero in every slot: run = half(run + alpha * slot sum).  C is
+// requested before anything else and converted once the first pair's loads have landed.
 template <int BI, int BJ, int WI, int WJ, int NSLOT, bool XK, bool YK, class CT, class DT, bool F16ACC>
 __global__ __launch_bounds__(WI *WJ * 64) __attribute__((amdgpu_waves_per_eu(2)))
 void k_gemm_pp64(tiled_params p)
@@ -554,8 +631,6 @@ void k_gemm_pp64(tiled_params p)
 
     const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
     const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);
-    const long xstep = XK ? KGRAN : (long)KGRAN * p.ldx;
-    const long ystep = YK ? KGRAN : (long)KGRAN * p.ldy;
     const unsigned xoff = xload::lane_offset(tid, (int)p.ldx);
     const unsigned yoff = yload::lane_offset(tid, (int)p.ldy);
 
@@ -591,7 +666,9 @@ void k_gemm_pp64(tiled_params p)
         return c;
     };
 
-    const int NP = p.K / KGRAN;
+    const int NP = (p.K + KGRAN - 1) / KGRAN;
+    // K tail: the last pair starts at K - 64; tail_skip of its k-values repeat the pair before
+    const int tail_skip = NP * KGRAN - p.K;
     const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
     int next = 0;          // next pair to request
     int wslot = 0;         // the slot it goes to
@@ -607,9 +684,9 @@ void k_gemm_pp64(tiled_params p)
     auto end_request = [&]() {
         next++;
         wslot = wslot + 1 == NSLOT ? 0 : wslot + 1;
-        const bool more = next < NP;
-        X += more ? xstep : 0;
-        Y += more ? ystep : 0;
+        const int kstep = next < NP - 1 ? KGRAN : next == NP - 1 ? KGRAN - tail_skip : 0;
+        X += XK ? (long)kstep : (long)kstep * p.ldx;
+        Y += YK ? (long)kstep : (long)kstep * p.ldy;
     };
 
     // fp16 accumulation: the C operand is requested first, as raw bits that no instruction touches
@@ -661,7 +738,7 @@ void k_gemm_pp64(tiled_params p)
             else fetch(std::false_type{});
         }
     }
-    // Prologue: the first NSLOT - 1 pairs.
+    // Prologue: the first NSLOT - 1 pairs are requested.
 #pragma unroll
     for (int s = 0; s < NSLOT - 1; s++) {
         begin_request();
@@ -669,7 +746,10 @@ void k_gemm_pp64(tiled_params p)
         (std::make_integer_sequence<int, LPAIR>{});
         end_request();
     }
-    wait_loads_and_barrier<0>();
+    // The loop starts when pair 0 (and the C operand, requested before it) has landed: the wait at the
+    // end of memory cluster p leaves NSLOT - 2 pairs in flight, so pair p + 1 has landed by then, the
+    // first time as every other.
+    wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
     float4_t cinit[F16ACC ? TI : 1][F16ACC ? TJ : 1];
     if constexpr (F16ACC) {
         auto convert = [&]<bool TRANS>(std::bool_constant<TRANS>) {
@@ -714,18 +794,14 @@ void k_gemm_pp64(tiled_params p)
         [&]<int... U>(std::integer_sequence<int, U...>) { ((fx[0][U] = fx[1][U] = xr.template read<U, 0>(lds)), ...); }(std::make_integer_sequence<int, TI>{});
         [&]<int... U>(std::integer_sequence<int, U...>) { ((fy[0][U] = fy[1][U] = yr.template read<U, 0>(lds + XBYTES)), ...); }(std::make_integer_sequence<int, TJ>{});
     }
-    // fp16 accumulation, for the tile MFMA number m of a k-step works on.
-    // RMODE 1, 2 (alpha == 1): the MFMAs accumulate onto the rounded running sum, which is rounded in
-    //     place once per slot; in the first slot (2) the sum meets half(beta * C) here.
+    // fp16 accumulation: rounding of tile t = a * TJ + b after its pair's MFMAs.
+    // RMODE 1 (alpha == 1): the accumulators start as half(beta * C), the MFMAs accumulate onto the
+    //     rounded running sum, and it is rounded in place once per slot.
     // RMODE 3 (any alpha): `cinit` is the running sum (a Float16 value held as Float32), the MFMA
     //     accumulators restart from zero in every slot and run = half(run + alpha * slot sum).
-    auto round_tile = [&]<int RMODE>(int m, std::integral_constant<int, RMODE>) {
-        const int a = m / TJ, b = serpentine_column(m, TJ);
+    auto round_tile = [&]<int RMODE>(int t, std::integral_constant<int, RMODE>) {
+        const int a = t / TJ, b = t % TJ;
         float4_t v = acc[a][b];
-        if constexpr (RMODE == 2) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] += cinit[a][b][e];
-        }
         if constexpr (RMODE == 3) {
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.alpha, v[e], cinit[a][b][e]);
@@ -767,11 +843,12 @@ void k_gemm_pp64(tiled_params p)
         rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
         __builtin_amdgcn_sched_barrier(0);
     };
-    // RMODE 0: fp32 sums over all of K; 1-3 (fp16 accumulation, see round_tile): each tile is rounded
-    // ROUND_LAG MFMAs after its last MFMA of the pair.
+    // ZERO (fp16 accumulation with alpha != 1): the accumulators restart from zero in every slot.
     constexpr int ROUND_LAG = 2;
-    auto compute_cluster = [&]<int RMODE>(std::integral_constant<int, RMODE>) {
+    auto tile_of_mfma = [](int m) { return m / TJ * TJ + serpentine_column(m, TJ); };
+    auto compute_cluster = [&]<bool ZERO>(std::bool_constant<ZERO>) {
         __builtin_amdgcn_sched_barrier(0);
+
 #pragma unroll
         for (int h = 0; h < 2; h++)
 #pragma unroll
@@ -779,16 +856,17 @@ void k_gemm_pp64(tiled_params p)
                 // serpentine order: every MFMA changes exactly one of its two operand fragments
                 const int a = m / TJ, b = serpentine_column(m, TJ);
                 if constexpr (!(MIW_PP_ABLATE & 4)) {
-                    if (RMODE == 3 && h == 0) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    if (ZERO && h == 0) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                     else acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], acc[a][b], 0, 0, 0);
                 }
-                if constexpr (RMODE != 0)
-                    if (h == 1 && m >= ROUND_LAG) round_tile(m - ROUND_LAG, std::integral_constant<int, RMODE>{});
+                // fp16 accumulation: a tile is rounded ROUND_LAG MFMAs after its last MFMA of the pair
+                if constexpr (F16ACC)
+                    if (h == 1 && m >= ROUND_LAG) round_tile(tile_of_mfma(m - ROUND_LAG), std::integral_constant<int, ZERO ? 3 : 1>{});
                 __builtin_amdgcn_sched_barrier(0);
             }
-        if constexpr (RMODE != 0)
+        if constexpr (F16ACC)
 #pragma unroll
-            for (int m = NTILE > ROUND_LAG ? NTILE - ROUND_LAG : 0; m < NTILE; m++) round_tile(m, std::integral_constant<int, RMODE>{});
+            for (int m = NTILE > ROUND_LAG ? NTILE - ROUND_LAG : 0; m < NTILE; m++) round_tile(tile_of_mfma(m), std::integral_constant<int, ZERO ? 3 : 1>{});
     };
 
     // Folding C (Float32 C laid out as D, alpha == 1): CPT MFMA tiles per cluster over the last
@@ -824,56 +902,99 @@ void k_gemm_pp64(tiled_params p)
         }
     };
     // One pair: memory cluster, barrier, compute cluster, barrier.  FS >= 0: fold cluster FS.
-    auto pair = [&]<int FS, int RMODE>(std::integral_constant<int, FS>, std::integral_constant<int, RMODE> rmode) {
+    // Zeroes the repeated k-values in the fragments of the shifted last pair.
+    auto mask_tail = [&]() {
+        const unsigned keep0 = tail_keep<0>(tail_skip), keep1 = tail_keep<1>(tail_skip);
+#pragma unroll
+        for (int a = 0; a < TI; a++) { tail_apply(fx[0][a], keep0); tail_apply(fx[1][a], keep1); }
+#pragma unroll
+        for (int b = 0; b < TJ; b++) { tail_apply(fy[0][b], keep0); tail_apply(fy[1][b], keep1); }
+    };
+    // FS >= 0: fold pair FS (always folds).  FS == -1: a pair that does not fold.  FS == -2: the last
+    // pair: its fragments are masked, and it is fold pair NFOLD - 1 when the launch folds C, which is
+    // decided here at run time, so that the last pair is one piece of code for both cases (two
+    // alternative pieces that each update all accumulators cost spills where they join).
+    auto fold_wait = [&]<int FS>(std::integral_constant<int, FS>) {
+        // Allowed to stay in flight: the ring loads of the NSLOT - 2 youngest clusters with the fold
+        // loads issued after them, and the fold loads of the cluster before those (younger than
+        // that cluster's ring loads, which must have landed).
+        constexpr int YOUNGER = (NSLOT - 2) * LPAIR + CPT * (FS + 1 < NSLOT - 1 ? FS + 1 : NSLOT - 1);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt((YOUNGER & 15) | (7 << 4) | (0 << 8) | ((YOUNGER >> 4) << 14));
+        asm volatile("" ::: "memory");
+    };
+    // RMODE: how the compute cluster rounds its sums (0: fp32 accumulation; 1, 3: see round_tile).
+    auto pair = [&]<int FS, int RMODE>(std::integral_constant<int, FS>, std::integral_constant<int, RMODE>) {
         memory_cluster();
         if constexpr (FS >= 0) {
             fold_request(std::integral_constant<int, FS>{});
             __builtin_amdgcn_sched_barrier(0);
-            // Allowed to stay in flight: the ring loads of the NSLOT - 2 youngest clusters with the fold
-            // loads issued after them, and the fold loads of the cluster before those (younger than
-            // that cluster's ring loads, which must have landed).
-            constexpr int YOUNGER = (NSLOT - 2) * LPAIR + CPT * (FS + 1 < NSLOT - 1 ? FS + 1 : NSLOT - 1);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_waitcnt((YOUNGER & 15) | (7 << 4) | (0 << 8) | ((YOUNGER >> 4) << 14));
-            asm volatile("" ::: "memory");
+            fold_wait(std::integral_constant<int, FS>{});
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (FS >= LAG) fold_add(std::integral_constant<int, FS - LAG>{});
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+        } else if constexpr (FS == -2 && CAN_FOLD) {
+            constexpr int LFS = NFOLD - 1;
+            if (fold_c) {
+                fold_request(std::integral_constant<int, LFS>{});
+                fold_wait(std::integral_constant<int, LFS>{});
+                fold_add(std::integral_constant<int, LFS - LAG>{});
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            } else {
+                wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
+            }
         } else {
             wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
         }
-        compute_cluster(rmode);
+        if constexpr (FS == -2) mask_tail();
+        compute_cluster(std::bool_constant<RMODE == 3>{});
         __builtin_amdgcn_s_barrier();
     };
     constexpr std::integral_constant<int, -1> no_fold{};
+    constexpr std::integral_constant<int, -2> last_pair{};
     constexpr std::integral_constant<int, 0> plain{};
 
     MIW_PP_STAMP(1)
     if (late_group) __builtin_amdgcn_s_barrier();
-    const int NPM = fold_c ? NP - NFOLD : NP;
+    // the loop runs the pairs that neither fold nor are the last one
+    const int NPM = fold_c ? NP - NFOLD : NP - 1;
     const bool separate_sum = F16ACC && p.alpha != 1.0f;
-    if (separate_sum) {
-        if constexpr (F16ACC)
-            for (int pr = 0; pr < NPM; pr++) pair(no_fold, std::integral_constant<int, 3>{});
+    if constexpr (F16ACC) {
+        // The running sum starts as half(beta * C): with alpha == 1 in the accumulators, which the MFMAs
+        // add onto; otherwise beside them.
+        constexpr std::integral_constant<int, 1> rolling{};
+        constexpr std::integral_constant<int, 3> separate{};
+        if (separate_sum) {
+            for (int pr = 0; pr < NPM; pr++) pair(no_fold, separate);
+            pair(last_pair, separate);
+        } else {
+#pragma unroll
+            for (int a = 0; a < TI; a++)
+#pragma unroll
+                for (int b = 0; b < TJ; b++) acc[a][b] = cinit[a][b];
+            for (int pr = 0; pr < NPM; pr++) pair(no_fold, rolling);
+            pair(last_pair, rolling);
+        }
     } else {
-        if (NPM > 0) pair(no_fold, std::integral_constant<int, F16ACC ? 2 : 0>{});
-        for (int pr = 1; pr < NPM; pr++) {
+        for (int pr = 0; pr < NPM; pr++) {
 #ifdef MIW_PP_TS
             if (pr == NPM / 2) MIW_PP_STAMP(2)
             if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
 #endif
-            pair(no_fold, std::integral_constant<int, F16ACC ? 1 : 0>{});
+            pair(no_fold, plain);
         }
-    }
-    MIW_PP_STAMP(9)
-    if constexpr (CAN_FOLD) {
-        if (fold_c) {
-            [&]<int... G>(std::integer_sequence<int, G...>) {
-                (pair(std::integral_constant<int, G>{}, plain), ...);
-            }(std::make_integer_sequence<int, NFOLD>{});
+        MIW_PP_STAMP(9)
+        if constexpr (CAN_FOLD) {
+            if (fold_c) {
+                [&]<int... G>(std::integer_sequence<int, G...>) {
+                    (pair(std::integral_constant<int, G>{}, plain), ...);
+                }(std::make_integer_sequence<int, NFOLD - 1>{});
+            }
         }
+        pair(last_pair, plain);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may outlive the workgroup's LDS
     if constexpr (CAN_FOLD) {

@@ -63,6 +63,9 @@ struct tiled_params {
     const half_t *Y;
     const void *C;
     void *D;
+    // K: any multiple of 16 from 64 up.  The kernels walk K in slots of 64; when 64 does not divide K
+    // the last slot is shifted back to end at K, and the k-values it repeats from the slot before
+    // (the first 64 * ceil(K / 64) - K of it) are zeroed in the fragments of both operands.
     int I, J, K;
     long ldx, ldy, ldc, ldd;
     long sx, sy, sc, sd;
@@ -224,6 +227,28 @@ struct frag_reader {
 
 __device__ inline float round_through_half(float v) { return (float)(half_t)v; }
 
+// K tail.  A lane's fragment of k-step H of a slot holds the 8 k-values 32 H + 8 q .. + 7 of the slot
+// (q = lane / 16), whichever operand layout it was read from.  In a last slot whose first `skip`
+// k-values (a multiple of 16) repeat the slot before, tail_keep is all ones for a lane whose values
+// count and zero otherwise.  The lane number is taken anew here: the mask is needed once per launch and
+// must not hold registers through the K loop.
+template <int H>
+__device__ inline unsigned tail_keep(int skip)
+{
+    const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    return 32 * H + 8 * (lane >> 4) >= skip ? 0xffffffffu : 0u;
+}
+// The masks are applied without a branch, in copies of the loop body that only the last pair runs
+// (a fragment that is changed on one side of a branch costs a second register set and a copy on the
+// other side, in every trip of the K loop).
+__device__ inline void tail_apply(half8_t &f, unsigned keep)
+{
+    uint4_t v = __builtin_bit_cast(uint4_t, f);
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] &= keep;
+    f = __builtin_bit_cast(half8_t, v);
+}
+
 // Ordinal of the direct-to-LDS load issued after MFMA m of a step of nmfma
 // matrix instructions that issues ndma loads, or -1.  The loads are spread
 // evenly over the step: a wavefront's load occupies the texture-address path
@@ -322,8 +347,6 @@ void k_gemm_tiled(tiled_params p)
 
     const half_t *X = p.X + bt * p.sx + (XK ? (long)i0 * p.ldx : (long)i0);
     const half_t *Y = p.Y + bt * p.sy + (YK ? (long)j0 * p.ldy : (long)j0);
-    const long xstep = XK ? KGRAN : (long)KGRAN * p.ldx;
-    const long ystep = YK ? KGRAN : (long)KGRAN * p.ldy;
     const unsigned xoff = xload::lane_offset(tid, (int)p.ldx);
     const unsigned yoff = yload::lane_offset(tid, (int)p.ldy);
 
@@ -381,7 +404,9 @@ void k_gemm_tiled(tiled_params p)
         }
     }
 
-    const int NP = p.K / KGRAN;  // slots' worth of K ("pairs" of steps)
+    const int NP = (p.K + KGRAN - 1) / KGRAN;  // slots' worth of K ("pairs" of steps)
+    // K tail: the last pair starts at K - 64; tail_skip of its k-values repeat the pair before
+    const int tail_skip = NP * KGRAN - p.K;
     const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
     constexpr int NLX = xload::NLOAD, NLY = yload::NLOAD, LPAIR = NLX + NLY;  // loads per thread and pair
     int next = 0;          // next pair to request
@@ -400,9 +425,9 @@ void k_gemm_tiled(tiled_params p)
     auto end_request = [&]() {
         next++;
         wslot = wslot + 1 == NSLOT ? 0 : wslot + 1;
-        const bool more = next < NP;
-        X += more ? xstep : 0;
-        Y += more ? ystep : 0;
+        const int kstep = next < NP - 1 ? KGRAN : next == NP - 1 ? KGRAN - tail_skip : 0;
+        X += XK ? (long)kstep : (long)kstep * p.ldx;
+        Y += YK ? (long)kstep : (long)kstep * p.ldy;
     };
     auto request_pair = [&]() {
         begin_request();
@@ -419,6 +444,14 @@ void k_gemm_tiled(tiled_params p)
         else f.y[U - TI] = yr.template read<U - TI, H>(xs + XBYTES);
     };
     constexpr int NUNIT = TI + TJ;
+    // Zeroes the repeated k-values in the fragments of half H of the shifted last pair.
+    auto mask_tail = [&]<int H>(frag_set<TI, TJ> &f, std::integral_constant<int, H>) {
+        const unsigned keep = tail_keep<H>(tail_skip);
+#pragma unroll
+        for (int a = 0; a < TI; a++) tail_apply(f.x[a], keep);
+#pragma unroll
+        for (int b = 0; b < TJ; b++) tail_apply(f.y[b], keep);
+    };
     // One pipeline step, in source order and pinned there: before MFMA m the
     // fragment unit m of the next step is fetched from LDS (all of them early
     // in the step, so they have landed long before it ends); the
@@ -547,35 +580,50 @@ void k_gemm_tiled(tiled_params p)
     // nothing new lands; its odd step reads another slot's stale bytes into
     // registers nobody uses.
     int rslot = 0;
-    const int NPM = fold_c ? NP - NCT : NP;
-    for (int pr = 0; pr < NPM; pr++) {
+    // MASK 1: the trip before the last pair's (its second step fetches the first half of the last pair);
+    // MASK 2: the last pair's own trip (its first step fetches the second half).
+    // G >= 0: the trip folds group G of C.  RT: whether it does is decided at run time (fold_c): the two
+    // trips that meet the last pair are one piece of code for launches that fold and launches that do
+    // not (two alternative pieces that each update all accumulators cost spills where they join).
+    auto trip = [&]<int MASK, int G, bool RT>(std::integral_constant<int, MASK>, std::integral_constant<int, G>, std::bool_constant<RT>) {
         step(f0, f1, rslot, second_half, dma_begin, dma_begin);
-        wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
+        if constexpr (MASK == 2) mask_tail(f1, second_half);
+        if constexpr (G >= 0) {
+            if (!RT || fold_c) wait_loads_and_barrier<(NSLOT - 2) * LPAIR + (G > 0 ? CPT : 0)>();
+            else wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
+        } else {
+            wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
+        }
         rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
+        if constexpr (G > 1)
+            if (!RT || fold_c) fold_fetch(std::integral_constant<int, G - 2>{});
+        __builtin_amdgcn_sched_barrier(0);
         begin_request();
         step(f1, f0, rslot, first_half, dma_begin, dma_end);
+        if constexpr (MASK == 1) mask_tail(f0, first_half);
         end_request();
-    }
+        if constexpr (G > 1)
+            if (!RT || fold_c) fold_add(std::integral_constant<int, G - 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (G >= 0)
+            if (!RT || fold_c) fold_request(std::integral_constant<int, G>{});
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    constexpr std::integral_constant<int, -1> no_group{};
+    // the loop runs the trips that neither fold nor meet the last pair
+    const int NPM = fold_c ? NP - NCT : NP >= 2 ? NP - 2 : 0;
+    for (int pr = 0; pr < NPM; pr++) trip(std::integral_constant<int, 0>{}, no_group, std::false_type{});
     if constexpr (CAN_FOLD) {
         if (fold_c) {
             [&]<int... G>(std::integer_sequence<int, G...>) {
-                (([&] {
-                     step(f0, f1, rslot, second_half, dma_begin, dma_begin);
-                     wait_loads_and_barrier<(NSLOT - 2) * LPAIR + (G > 0 ? CPT : 0)>();
-                     rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
-                     if constexpr (G > 1) fold_fetch(std::integral_constant<int, G - 2>{});
-                     __builtin_amdgcn_sched_barrier(0);
-                     begin_request();
-                     step(f1, f0, rslot, first_half, dma_begin, dma_end);
-                     end_request();
-                     if constexpr (G > 1) fold_add(std::integral_constant<int, G - 2>{});
-                     __builtin_amdgcn_sched_barrier(0);
-                     fold_request(std::integral_constant<int, G>{});
-                     __builtin_amdgcn_sched_barrier(0);
-                 }()),
-                 ...);
-            }(std::make_integer_sequence<int, NCT>{});
+                (trip(std::integral_constant<int, 0>{}, std::integral_constant<int, G>{}, std::false_type{}), ...);
+            }(std::make_integer_sequence<int, NCT - 2>{});
         }
+        if (NP >= 2) trip(std::integral_constant<int, 1>{}, std::integral_constant<int, NCT - 2>{}, std::true_type{});
+        trip(std::integral_constant<int, 2>{}, std::integral_constant<int, NCT - 1>{}, std::true_type{});
+    } else {
+        if (NP >= 2) trip(std::integral_constant<int, 1>{}, no_group, std::false_type{});
+        trip(std::integral_constant<int, 2>{}, no_group, std::false_type{});
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may outlive the workgroup's LDS
     if constexpr (CAN_FOLD) {

@@ -53,6 +53,31 @@ def synchronize(stream=None):
     _lib.check(_lib.load().miw_sync(_stream_handle(stream)))
 
 
+def warpsize(dev=None):
+    """Lanes of a wavefront on the device (CUDAdrv.warpsize): 64 on gfx950; read from the device once the
+    library is initialised, `dev` being a device_info() dict or None for the current device."""
+    if isinstance(dev, dict):
+        return int(dev["wave_size"])
+    info = _lib.DeviceInfo()
+    if _lib.load().miw_device_info_get(ctypes.byref(info)) == 0:
+        return int(info.wave_size)
+    return WAVEFRONT
+
+
+def nextwarp(dev, threads):
+    """The nearest number of threads >= `threads` that is a multiple of the device's wavefront size
+    (src/execution.jl:418-421)."""
+    ws = warpsize(dev)
+    return threads + (ws - threads % ws) % ws
+
+
+def prevwarp(dev, threads):
+    """The nearest number of threads <= `threads` that is a multiple of the device's wavefront size
+    (src/execution.jl:423-426)."""
+    ws = warpsize(dev)
+    return threads - threads % ws
+
+
 def cudaconvert(arg):
     """Host object -> what the kernel sees (src/execution.jl:119-141)."""
     if isinstance(arg, DeviceArray):

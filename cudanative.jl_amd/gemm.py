@@ -79,6 +79,13 @@ def splitk_static_capacity():
     return _lib.load().miw_gemm_splitk_static_capacity()
 
 
+def splitk_static_plan(desc, splits=0):
+    """(slices, bytes of the static workspace) gemm_splitk_static will use; touches no device."""
+    n, nbytes = ctypes.c_int(), ctypes.c_size_t()
+    _lib.check(_lib.load().miw_gemm_splitk_static_plan(ctypes.byref(desc), splits, ctypes.byref(n), ctypes.byref(nbytes)))
+    return n.value, nbytes.value
+
+
 def gemm_bench(A, B, C, D, desc, warmup=5, iters=20, stream=None):
     """Per-launch durations in milliseconds, HIP events on the launch stream."""
     ms = (ctypes.c_float * iters)()
@@ -127,3 +134,13 @@ def acc_chunk(desc):
     v = ctypes.c_int()
     _lib.check(_lib.load().miw_gemm_acc_chunk(ctypes.byref(desc), ctypes.byref(v)))
     return v.value
+
+
+def resolve(A, B, C, D, desc):
+    """(variant, acc_chunk) of the launch gemm(A, B, C, D, desc) makes first: the same checks and plan on
+    the real operand addresses (alignment, C sharing memory with D), without a launch.  acc_chunk is 0
+    with Float32 accumulation."""
+    v, chunk = ctypes.c_int(), ctypes.c_int()
+    _lib.check(_lib.load().miw_gemm_resolve(ctypes.byref(desc), _ptr(A), _ptr(B), _ptr(C), _ptr(D), ctypes.byref(v),
+                                            ctypes.byref(chunk)))
+    return v.value, chunk.value

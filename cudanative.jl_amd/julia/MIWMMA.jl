@@ -30,7 +30,7 @@ module MIWMMA
 
 export DeviceBuffer, DevicePtr, AS, WMMA, @hip, gemm!, gemm_splitk!, gemm_splitk_static!, synchronize, MIWError,
        HostKernel, hipfunction, CodeObject, kernel, registers, memory, maxthreads, launch_configuration,
-       Stream, device_info
+       Stream, device_info, warpsize, nextwarp, prevwarp, mem_info
 
 const libmiwmma = get(ENV, "MIWMMA_LIB", joinpath(@__DIR__, "..", "libmiwmma.so"))
 
@@ -77,6 +77,25 @@ function device_info()
     return (name=cstring(d.name), arch=cstring(d.arch), cu_count=Int(d.cu_count), wave_size=Int(d.wave_size),
             clock_mhz=Int(d.clock_mhz), lds_per_block=Int(d.lds_per_block), hbm_bytes=Int(d.hbm_bytes),
             peak_f16_tflops=d.peak_f16_tflops)
+end
+
+"Lanes of a wavefront (CUDAdrv.warpsize): 64 on gfx950.  `dev` is what device_info() returns."
+warpsize(dev=device_info()) = dev.wave_size
+
+"""
+    nextwarp(dev, threads)
+    prevwarp(dev, threads)
+
+The next or previous nearest number of threads that is a multiple of the wavefront size of the
+device (src/execution.jl:418-426).
+"""
+function nextwarp(dev, threads::Integer)
+    ws = warpsize(dev)
+    return threads + (ws - threads % ws) % ws
+end
+function prevwarp(dev, threads::Integer)
+    ws = warpsize(dev)
+    return threads - rem(threads, ws)
 end
 
 # ---------------------------------------------------------------------------- streams -----
@@ -195,6 +214,13 @@ function Base.copyto!(dst::DeviceBuffer{T}, src::DeviceBuffer{T}) where {T}
     check(ccall((:miw_memcpy_d2d, libmiwmma), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t), dst.ptr, src.ptr, length(src) * sizeof(T)))
     return dst
 end
+"(free, total) bytes of device memory."
+function mem_info()
+    f, t = Ref{Csize_t}(0), Ref{Csize_t}(0)
+    check(ccall((:miw_mem_info, libmiwmma), Cint, (Ptr{Csize_t}, Ptr{Csize_t}), f, t))
+    return Int(f[]), Int(t[])
+end
+
 function Base.fill!(a::DeviceBuffer{T}, byte::UInt8) where {T}
     check(ccall((:miw_memset, libmiwmma), Cint, (Ptr{Cvoid}, Cint, Csize_t), a.ptr, byte, length(a) * sizeof(T)))
     return a
@@ -692,6 +718,15 @@ function acc_chunk(desc::GemmDesc)
     return Int(v[])
 end
 
+"(variant, acc_chunk) of the first launch gemm! makes for these operands (alignment and a C that is D count); no launch."
+function gemm_resolve(desc::GemmDesc, A::DeviceBuffer, B::DeviceBuffer, C::Union{DeviceBuffer,Nothing}, D::DeviceBuffer)
+    v, chunk = Ref{Cint}(0), Ref{Cint}(0)
+    GC.@preserve A B C D check(ccall((:miw_gemm_resolve, libmiwmma), Cint,
+        (Ptr{GemmDesc}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cint}, Ptr{Cint}),
+        Ref(desc), A.ptr, B.ptr, C === nothing ? C_NULL : C.ptr, D.ptr, v, chunk))
+    return Int(v[]), Int(chunk[])
+end
+
 "(slices, workspace bytes) of a split-K launch of this problem (splits = 0: chosen by the library)."
 function splitk_workspace(desc::GemmDesc, splits::Integer=0)
     n, bytes = Ref{Cint}(0), Ref{Csize_t}(0)
@@ -713,6 +748,14 @@ function gemm_splitk!(D::DeviceBuffer{DT}, A::DeviceBuffer{Float16}, B::DeviceBu
 end
 
 splitk_static_capacity() = Int(ccall((:miw_gemm_splitk_static_capacity, libmiwmma), Csize_t, ()))
+
+"(slices, bytes of the static workspace) gemm_splitk_static! will use; touches no device."
+function splitk_static_plan(desc::GemmDesc, splits::Integer=0)
+    n, bytes = Ref{Cint}(0), Ref{Csize_t}(0)
+    check(ccall((:miw_gemm_splitk_static_plan, libmiwmma), Cint, (Ptr{GemmDesc}, Cint, Ptr{Cint}, Ptr{Csize_t}),
+                Ref(desc), splits, n, bytes))
+    return Int(n[]), Int(bytes[])
+end
 
 "Split-K GEMM through the library's static device workspace: allocates nothing; calls that overlap on one GPU race."
 function gemm_splitk_static!(D::DeviceBuffer{DT}, A::DeviceBuffer{Float16}, B::DeviceBuffer{Float16},

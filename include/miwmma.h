@@ -101,6 +101,9 @@ int miw_memcpy_h2d(void *dst, const void *src_host, size_t bytes);
 int miw_memcpy_d2h(void *dst_host, const void *src, size_t bytes);
 int miw_memcpy_d2d(void *dst, const void *src, size_t bytes);
 int miw_memset(void *dst, int byte, size_t bytes);
+/* Free and total device memory in bytes: what the OOM -> GC.gc() -> retry path of the allocator
+   (src/array.jl:23-29) consults, and what a test of an allocation-free call compares. */
+int miw_mem_info(size_t *free_bytes, size_t *total_bytes);
 
 /* stream= keyword of @cuda (src/execution.jl:59-63); synchronize() */
 int miw_stream_create(void **out);
@@ -234,8 +237,17 @@ typedef struct miw_gemm_part {
     int64_t m, n, k;      /* its sizes */
 } miw_gemm_part;
 int miw_gemm_plan(const miw_gemm_desc *desc, int in_place, miw_gemm_part *parts, int capacity, int *count);
-/* acc_chunk miw_gemm would use for this descriptor (fp16 accumulate only). */
+/* acc_chunk miw_gemm would use for this descriptor (fp16 accumulate only).  Like
+   miw_gemm_pick_variant it sees no pointers and assumes 16-byte aligned operands with C and D
+   apart; operands that are not (or a C that is D, with M or N no whole number of tiles) can send
+   miw_gemm to another kernel with another acc_chunk: miw_gemm_resolve answers for the real ones. */
 int miw_gemm_acc_chunk(const miw_gemm_desc *desc, int *acc_chunk);
+/* What miw_gemm(desc, A, B, C, D, ...) will run, from the same checks and plan but without a
+   launch: *variant = the variant of its first launch, *acc_chunk = the k-values between two
+   roundings of the Float16 running sum (0 with Float32 accumulation).  Either output may be null.
+   No counterpart in the reference (its mma chain always rounds once per 16 x 16 x 16 tile). */
+int miw_gemm_resolve(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, const void *D,
+                     int *variant, int *acc_chunk);
 
 /* Split-K form of miw_gemm for problems with few output tiles and a long K: the chain of mma
    calls over K (docs/src/device/wmma.md:51-52) is cut into `splits` equal slices (each a multiple
@@ -252,18 +264,22 @@ int miw_gemm_splitk_workspace(const miw_gemm_desc *desc, int splits, int *splits
 int miw_gemm_splitk(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
                     void *workspace, size_t workspace_bytes, void *stream);
 
-/* miw_gemm_splitk for callers that cannot allocate device memory (code under HIP graph capture,
-   tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+/* miw_gemm_splitk for callers that cannot allocate device memory (tight serving loops, harnesses
+   that forbid hipMalloc).  It has no counterpart in the reference.
    Same kernels and results as miw_gemm_splitk, with the slices going through a workspace that is
    part of the library's device code: miw_gemm_splitk_static_capacity() bytes (32 MiB) that every
    GPU the library runs on holds until the process ends.  It calls no hipMalloc, hipFree or other
    allocating routine, and refuses (MIW_ERR_UNSUPPORTED) a problem whose splits * m * n * 4 bytes
    exceed the capacity.  All calls on one GPU share that GPU's workspace: calls that overlap on one
    GPU (two streams, two host threads) race; calls on one stream are ordered and safe.  Nothing in
-   the workspace needs clearing: the first pass writes every element the second pass reads. */
+   the workspace needs clearing: the first pass writes every element the second pass reads.
+   splits = 0 chooses among the slice counts whose partial products fit the capacity (one slice, the
+   plain launch, always does).  miw_gemm_splitk_static_plan reports the count and the bytes of the
+   static workspace a call will use, without touching the device. */
 int miw_gemm_splitk_static(const miw_gemm_desc *desc, const void *A, const void *B, const void *C, void *D, int splits,
                            void *stream);
 size_t miw_gemm_splitk_static_capacity(void);
+int miw_gemm_splitk_static_plan(const miw_gemm_desc *desc, int splits, int *splits_out, size_t *bytes);
 
 /* warmup untimed launches, then iters launches each bracketed by HIP events on
    `stream`; ms_each[i] receives launch i's duration in milliseconds. */

@@ -18,18 +18,10 @@ def load_package():
     spec_b = importlib.util.spec_from_file_location("_miw_build", os.path.join(PKG_DIR, "build.py"))
     b = importlib.util.module_from_spec(spec_b)
     spec_b.loader.exec_module(b)
-    lib_path = os.path.join(PKG_DIR, "libmiwmma.so")
-    stale = False
-    if os.path.exists(lib_path):
-        # the library carries the hash of the sources it was built from
-        import ctypes
-        probe = ctypes.CDLL(lib_path)
-        try:
-            probe.miw_build_id.restype = ctypes.c_char_p
-            stale = probe.miw_build_id().decode() != b.source_id()
-        except AttributeError:      # a library from before the hash existed
-            stale = True
-    if stale or not os.path.exists(lib_path):
+    # The library carries the hash of the sources it was built from.  It is read from the file, not by
+    # loading the library: a binary loaded here would stay this process's libmiwmma.so even after a
+    # rebuild at the same path, and the tests would then run against the stale kernels.
+    if b.built_id() != b.source_id():
         # nothing built yet, or built from other sources: build once (hipcc cross-compiles without a GPU)
         b.build()
     spec = importlib.util.spec_from_file_location(name, os.path.join(PKG_DIR, "__init__.py"),
@@ -37,6 +29,10 @@ def load_package():
     mod = importlib.util.module_from_spec(spec)
     sys.modules[name] = mod
     spec.loader.exec_module(mod)
+    if not os.environ.get("MIWMMA_LIB"):
+        loaded = mod._lib.load().miw_build_id().decode()
+        if loaded != b.source_id():
+            raise RuntimeError("libmiwmma.so in this process has build id %s, the sources have %s" % (loaded, b.source_id()))
     return mod
 
 

@@ -67,6 +67,10 @@ def _variants(gpu):
     return gpu.GEMM.variants()
 
 
+def _vid(gpu, name):
+    return [v["id"] for v in gpu.GEMM.variants() if v["name"] == name][0]
+
+
 def _restricted(v):
     """Variants that serve only part of the problem space (operand layouts, K extent): _run checks that
     the library refuses the rest and returns None."""
@@ -153,17 +157,17 @@ def test_tiled_variants_agree_bitwise(gpu, orc):
     for o in outs[1:]:
         assert np.array_equal(o.view(np.uint32), outs[0].view(np.uint32))
     # twice the same launch: deterministic
-    assert np.array_equal(_run(gpu, orc, g, A, B, C, variant=1).view(np.uint32), outs[0].view(np.uint32))
+    assert np.array_equal(_run(gpu, orc, g, A, B, C, variant=_vid(gpu, "tile256x128_w4x2")).view(np.uint32), outs[0].view(np.uint32))
 
 
-# K long enough (more than 16 LDS slots' worth) for the 8-wavefront 256x256, 256x128 and 128x256
-# kernels to add C into their accumulators during the last trips of the loop instead of in the epilogue.
+# K long enough (more than 16 LDS slots' worth) for the 8-wavefront 256x128 and 128x256 kernels and the
+# ping-pong kernels to add C into their accumulators during the last trips of the loop instead of in the epilogue.
 
 @pytest.mark.parametrize("al,bl,dl", itertools.product((0, 1), repeat=3))
 @pytest.mark.parametrize("K", [17 * 64, 20 * 64])
 def test_c_folded_into_the_loop_exact_on_integers(gpu, orc, al, bl, dl, K):
     folding = [v for v in _variants(gpu) if v["waves"][0] * v["waves"][1] == 8 and v["stages"] <= 3]
-    assert [v["block"][:2] for v in folding if not v["pingpong"]] == [(256, 256), (256, 128), (128, 256)]
+    assert [v["block"][:2] for v in folding if not v["pingpong"]] == [(256, 128), (128, 256)]
     assert any(v["pingpong"] for v in folding)
     for v in folding:
         g = orc.GemmDesc(M=512, N=256, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, beta=-2.0)
@@ -182,25 +186,26 @@ def test_c_folded_into_the_loop_matches_the_epilogue_path(gpu, orc):
                      stride_a=264 * 1600 + 8, stride_b=1608 * 512, stride_c=272 * 512 + 16, stride_d=260 * 512)
     A, B, C = _inputs(orc, g, 77)
     ref = orc.gemm_f64(g, A, B, C)
-    folded = _run(gpu, orc, g, A, B, C, variant=1, prefill=5.0)
+    fold = _vid(gpu, "tile256x128_w4x2")
+    folded = _run(gpu, orc, g, A, B, C, variant=fold, prefill=5.0)
     assert orc.normalized_error(g, folded, ref) <= TIGHT_F32
-    for v in (3, 4):
-        assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C, variant=v, prefill=5.0), ref) <= TIGHT_F32
-    other = _run(gpu, orc, g, A, B, C, variant=2, prefill=5.0)           # 4 wavefronts: C in the epilogue
+    for name in ("tile128x256_w2x4", "tile256x256_pingpong", "tile256x128_pingpong"):
+        assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C, variant=_vid(gpu, name), prefill=5.0), ref) <= TIGHT_F32, name
+    other = _run(gpu, orc, g, A, B, C, variant=_vid(gpu, "tile256x256_w2x2"), prefill=5.0)   # 4 wavefronts: C in the epilogue
     assert orc.normalized_error(g, other, ref) <= TIGHT_F32
     assert np.max(np.abs(folded.astype(np.float64) - other)) <= 4e-7 * np.abs(ref).max()   # padding: 5.0 in both
     assert np.count_nonzero(folded == 5.0) >= (260 - 256) * 512 * 2
     # alpha != 1 and a C stored across D take the epilogue path of the same kernel
     g2 = orc.GemmDesc(M=256, N=256, K=1600, alpha=0.5, beta=0.75)
     A, B, C = _inputs(orc, g2, 78)
-    assert orc.normalized_error(g2, _run(gpu, orc, g2, A, B, C, variant=1), orc.gemm_f64(g2, A, B, C)) <= TIGHT_F32
+    assert orc.normalized_error(g2, _run(gpu, orc, g2, A, B, C, variant=fold), orc.gemm_f64(g2, A, B, C)) <= TIGHT_F32
     g3 = orc.GemmDesc(M=256, N=256, K=1600, c_layout=orc.ROW, beta=0.75)
     A, B, C = _inputs(orc, g3, 79)
-    assert orc.normalized_error(g3, _run(gpu, orc, g3, A, B, C, variant=1), orc.gemm_f64(g3, A, B, C)) <= TIGHT_F32
+    assert orc.normalized_error(g3, _run(gpu, orc, g3, A, B, C, variant=fold), orc.gemm_f64(g3, A, B, C)) <= TIGHT_F32
     # half C with float accumulation is not folded (the staging loads move 16 bytes per lane)
     g4 = orc.GemmDesc(M=256, N=256, K=1600, c_type=orc.F16, beta=0.75)
     A, B, C = _inputs(orc, g4, 80)
-    assert orc.normalized_error(g4, _run(gpu, orc, g4, A, B, C, variant=1), orc.gemm_f64(g4, A, B, C)) <= TIGHT_F32
+    assert orc.normalized_error(g4, _run(gpu, orc, g4, A, B, C, variant=fold), orc.gemm_f64(g4, A, B, C)) <= TIGHT_F32
 
 
 def test_c_and_d_may_be_one_buffer(gpu, orc):
@@ -264,14 +269,27 @@ def test_seeded_sweep_over_variants_layouts_and_scalars(gpu, orc):
 
 
 def test_ragged_sizes_fall_back_to_fragment_ops(gpu, orc):
-    # multiples of 16 that no LDS tile divides, padded leading dimensions, odd batch strides
-    g = orc.GemmDesc(M=80, N=112, K=176, lda=88, ldb=200, ldc=96, ldd=104, batch=3,
-                     stride_a=88 * 176 + 8, stride_b=200 * 112 + 24, stride_c=96 * 112, stride_d=104 * 112 + 40)
-    assert gpu.GEMM.variants()[gpu.GEMM.pick_variant(gpu.GEMM.make_desc(80, 112, 176)) - 1]["fragment_ops"]
+    # an extent smaller than every LDS tile, padded leading dimensions, odd batch strides
+    g = orc.GemmDesc(M=48, N=112, K=176, lda=56, ldb=200, ldc=64, ldd=72, batch=3,
+                     stride_a=56 * 176 + 8, stride_b=200 * 112 + 24, stride_c=64 * 112, stride_d=72 * 112 + 40)
+    assert gpu.GEMM.variants()[gpu.GEMM.pick_variant(gpu.GEMM.make_desc(48, 112, 176)) - 1]["fragment_ops"]
     A, B, C = _inputs(orc, g, 31)
     D = _run(gpu, orc, g, A, B, C, prefill=-5.0)
     assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
     # padding between columns and between batches is never written
+    gr = g.resolved()
+    Dm = D.reshape(-1)
+    for bt in range(3):
+        blk = Dm[bt * gr.stride_d: bt * gr.stride_d + 72 * 112].reshape(112, 72)
+        assert np.all(blk[:, 48:] == -5.0)
+        assert np.all(Dm[bt * gr.stride_d + 72 * 112:(bt + 1) * gr.stride_d] == -5.0)
+    # the same with extents of one tile and a bit and K = 128 + 48: the smallest LDS tile, edge tiles and last slot shifted back
+    g = orc.GemmDesc(M=80, N=112, K=176, lda=88, ldb=200, ldc=96, ldd=104, batch=3,
+                     stride_a=88 * 176 + 8, stride_b=200 * 112 + 24, stride_c=96 * 112, stride_d=104 * 112 + 40)
+    assert not gpu.GEMM.variants()[gpu.GEMM.pick_variant(gpu.GEMM.make_desc(80, 112, 176)) - 1]["fragment_ops"]
+    A, B, C = _inputs(orc, g, 32)
+    D = _run(gpu, orc, g, A, B, C, prefill=-5.0)
+    assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
     gr = g.resolved()
     Dm = D.reshape(-1)
     for bt in range(3):
@@ -293,9 +311,10 @@ def _plan(gpu, orc, g, in_place=False):
 @pytest.mark.parametrize("al,bl,cl,dl", [(1, 1, 1, 1), (0, 1, 1, 0), (1, 0, 0, 1), (0, 0, 0, 0)])
 def test_ragged_sizes_cut_into_tiled_parts_exact_on_integers(gpu, orc, al, bl, cl, dl):
     """Sizes that are multiples of 16 but of no LDS tile: the tiled kernels shift their edge tiles back
-    so that they end at the edge, and the last k-values beyond a multiple of 64 go through the
-    fragment-op kernel as a second launch.  On small integers every part is exact, so the result must
-    equal the oracle bit for bit whatever the cuts, and nothing outside D's extent may be written."""
+    so that they end at the edge, and their last slot of 64 k-values back so that it ends at K (the
+    k-values it repeats are zeroed in the fragments).  On small integers every part is exact, so the
+    result must equal the oracle bit for bit whatever the cuts, and nothing outside D's extent may be
+    written."""
     frag = gpu.GEMM.variants()[-1]["id"]
     for n, (M, N, K, kw) in enumerate([(1040, 1104, 1040, {}),                       # ragged in m, n and k
                                        (592, 656, 2064, dict(alpha=-2.0, beta=0.5)),
@@ -307,7 +326,7 @@ def test_ragged_sizes_cut_into_tiled_parts_exact_on_integers(gpu, orc, al, bl, c
         g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl,
                          lda=(K if al == orc.ROW else M) + pad, ldd=(N if dl == orc.ROW else M) + 2 * pad, **kw)
         parts = _plan(gpu, orc, g)
-        assert any(q["variant"] != frag for q in parts) and (K % 64 == 0 or len(parts) >= 2), (M, N, K, parts)
+        assert all(q["variant"] != frag and q["k0"] == 0 and q["k"] == K for q in parts), (M, N, K, parts)
         # the parts cover D and the K extent
         cover = np.zeros((M, N), dtype=np.int64)
         for q in parts:
@@ -362,20 +381,67 @@ def test_edge_tiles_shifted_back_every_variant(gpu, orc, al, bl, dl):
     assert e.value.code == gpu._lib.ERR_UNSUPPORTED
 
 
+@pytest.mark.parametrize("al,bl,dl", itertools.product((0, 1), repeat=3))
+def test_k_tail_every_variant(gpu, orc, al, bl, dl):
+    """K = 64 q + r, r = 16, 32, 48: every tiled variant shifts its last slot back to end at K and zeroes
+    the k-values the slot repeats.  Bit-exact on integers, with Float32 accumulation (K short, and long
+    enough for the kernels that fold C into the last trips of the loop) and with Float16 accumulation
+    (whose chunked model then ends on a chunk of r k-values)."""
+    for v in _variants(gpu):
+        if v["fragment_ops"]:
+            continue
+        bm, bn = v["block"][:2]
+        big = max(bm, bn)
+        for K in (64 + 16, 128 + 32, 192 + 48, 64 * 34 + 16 * (1 + v["id"] % 3)):
+            g = orc.GemmDesc(M=big, N=2 * big if K < 1024 else big, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, beta=-1.0)
+            A, B, C = _inputs(orc, g, 1500 + K + v["id"], ints=True)
+            D = _run(gpu, orc, g, A, B, C, variant=v["id"])
+            assert D is not None and np.array_equal(D, orc.gemm(g, A, B, C)), (v["name"], al, bl, dl, K)
+        if not v["f16_accumulate"]:
+            continue
+        for K in (64 + 48, 192 + 16):
+            g = orc.GemmDesc(M=big, N=big, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, c_type=orc.F16, d_type=orc.F16)
+            A, B, C = _inputs(orc, g, 1600 + K + v["id"], ints=True)        # |sums| < 2048: exact in half
+            D = _run(gpu, orc, g, A, B, C, variant=v["id"], acc_type=F16)
+            assert np.array_equal(D, orc.gemm_f16acc(g, 64, A, B, C)), (v["name"], al, bl, dl, K)
+
+
+def test_k_tail_random_data(gpu, orc):
+    """Uniform data, K = 64 q + r on the kernels miw_gemm picks: Float32 accumulation against float64, a
+    Float16 D, and Float16 accumulation against the chunked model (chunks of 64, the last one of r)."""
+    frag = gpu.GEMM.variants()[-1]["id"]
+    for n, (M, N, K, kw) in enumerate([(512, 512, 4112, {}), (256, 768, 1072, dict(a_layout=orc.ROW, alpha=0.5, beta=-1.5)),
+                                       (1024, 256, 2096, dict(b_layout=orc.ROW, d_type=orc.F16))]):
+        g = orc.GemmDesc(M=M, N=N, K=K, **kw)
+        assert [q["k"] for q in _plan(gpu, orc, g)] == [K] and _plan(gpu, orc, g)[0]["variant"] != frag
+        A, B, C = _inputs(orc, g, 1700 + n)
+        err = orc.normalized_error(g, _run(gpu, orc, g, A, B, C), orc.gemm_f64(g, A, B, C))
+        assert err <= (6e-4 if g.d_type == orc.F16 else TIGHT_F32), (M, N, K, err)
+    g = orc.GemmDesc(M=512, N=512, K=1040, c_type=orc.F16, d_type=orc.F16)
+    A, B, C = _inputs(orc, g, 1710, lo=-0.5, hi=0.5, clo=-0.1, chi=0.1)
+    desc = gpu.GEMM.make_desc(512, 512, 1040, c_type=F16, d_type=F16, acc_type=F16)
+    assert gpu.GEMM.acc_chunk(desc) == 64 and gpu.GEMM.pick_variant(desc) != frag
+    D = _run(gpu, orc, g, A, B, C, acc_type=F16)
+    _assert_matches_model(D, orc.gemm_f16acc(g, 64, A, B, C))
+    assert orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C)) <= TOL_F16ACC
+
+
 def test_ragged_sizes_random_data_and_in_place(gpu, orc):
-    """Random data against float64 (the k tail adds one Float32 rounding per element), and the in-place
-    case: with C and D one buffer the windows must not overlap what an earlier part stored."""
+    """Random data against float64, and the in-place case: with C and D one buffer the windows must
+    not overlap what an earlier part stored."""
     frag = gpu.GEMM.variants()[-1]["id"]
     g = orc.GemmDesc(M=1104, N=1040, K=2064, alpha=0.75, beta=-1.25)
-    assert len(_plan(gpu, orc, g)) >= 2
+    assert all(q["variant"] != frag for q in _plan(gpu, orc, g))
     A, B, C = _inputs(orc, g, 1300)
     assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
-    # Float16 D: the k extent is not cut (a second rounding to Float16 would show)
+    # Float16 D (one rounding to Float16, whatever K is)
     g = orc.GemmDesc(M=2064, N=80, K=1024, d_type=orc.F16)
     A, B, C = _inputs(orc, g, 1310)
     assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C), orc.gemm_f64(g, A, B, C)) <= 6e-4
     g = orc.GemmDesc(M=1104, N=1040, K=1040, d_type=orc.F16)
-    assert [q["variant"] for q in _plan(gpu, orc, g)] == [frag]
+    assert all(q["variant"] != frag for q in _plan(gpu, orc, g))
+    A, B, C = _inputs(orc, g, 1311)
+    assert orc.normalized_error(g, _run(gpu, orc, g, A, B, C), orc.gemm_f64(g, A, B, C)) <= 6e-4
     # in place: disjoint parts only
     for M, N, K in ((2112, 2112, 1040), (2112 + 16, 2112, 1024)):
         g = orc.GemmDesc(M=M, N=N, K=K, beta=0.5)
@@ -457,7 +523,7 @@ def test_seeded_sweep_over_ragged_sizes(gpu, orc):
         else:
             err = orc.normalized_error(g, D, orc.gemm_f64(g, A, B, C))
             assert err <= (TIGHT_F32 if dt == orc.F32 else 6e-4), (case, err)
-    assert cut >= 2 and forced >= 30 and inplace >= 5, (cut, forced, inplace)
+    assert forced >= 30 and inplace >= 5, (cut, forced, inplace)
 
 
 @pytest.mark.parametrize("al,bl,dl", itertools.product((0, 1), repeat=3))
@@ -517,7 +583,8 @@ def test_thin_problems_share_a_tile_between_wavefronts(gpu, orc, al, bl, cl, dl)
                                        (64, 4096, 2064, dict(d_type=orc.F16, c_type=orc.F16))]):   # 16 wavefronts x 4 tiles: 64 KiB of partial sums
         g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl,
                          ldd=(N if dl == orc.ROW else M) + 8, **kw)
-        assert [q["variant"] for q in _plan(gpu, orc, g)][-1] == frag
+        if min(M, N) < 64:          # thinner than every LDS tile
+            assert [q["variant"] for q in _plan(gpu, orc, g)] == [frag]
         A, B, C = _inputs(orc, g, 1600 + n, ints=True)
         want = orc.gemm(g, A, B, C)
         D = _run(gpu, orc, g, A, B, C if g.use_c else None, prefill=7.0)

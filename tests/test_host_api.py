@@ -187,7 +187,7 @@ def test_abi_rejects_bad_arguments_without_touching_the_gpu(miw):
     assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_VALUE
     d = G.make_desc(64, 64, 64, batch=0)
     assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_INVALID_VALUE
-    d = G.make_desc(80, 64, 64, variant=1)                     # not divisible by the 256x256 tile
+    d = G.make_desc(80, 64, 64, variant=1)                     # smaller than the variant's tile
     assert lib.miw_gemm(ctypes.byref(d), p, p, p, p, None) == L.ERR_UNSUPPORTED
     k = ctypes.c_void_p()
     assert lib.miw_kernel_lookup(b"no_such_kernel", ctypes.byref(k)) == L.ERR_NOT_FOUND
@@ -231,13 +231,13 @@ def test_gemm_plan_covers_the_problem(miw):
                 sub = G.make_desc(q["m"], q["n"], q["k"], a_layout=layouts[case & 1], b_layout=layouts[(case >> 1) & 1],
                                   d_layout=layouts[(case >> 2) & 1], c_layout=layouts[(case >> 2) & 1], d_type=dt,
                                   lda=desc.lda or (K if case & 1 else M), batch=1 + case % 3)
-                assert q["k"] % 64 == 0 and G.variant_supports(sub, q["variant"]), (M, N, K, q)
+                assert q["k"] >= 64 and G.variant_supports(sub, q["variant"]), (M, N, K, q)
                 bm, bn = vs[q["variant"] - 1]["block"][:2]
                 tm, tn = (bn, bm) if (case >> 2) & 1 else (bm, bn)
                 if in_place:                      # whole tiles only
                     assert q["m"] % tm == 0 and q["n"] % tn == 0, (M, N, K, q)
-            if q["k0"] > 0:                       # a k tail: Float32 D only, over the part of D its body covered
-                assert dt == np.float32 and q["variant"] == frag and q["k0"] % 64 == 0 and q["k0"] + q["k"] == K
+            # K is never cut: the tiled kernels shift their last slot of 64 k-values back to end at K
+            assert q["k0"] == 0 and q["k"] == K, (M, N, K, q)
         assert cover.min() >= K, (M, N, K, in_place, parts)
         if in_place:
             assert first.min() == 1 and first.max() == 1 and cover.max() == K, (M, N, K, parts)
@@ -247,7 +247,11 @@ def test_gemm_plan_covers_the_problem(miw):
     d = G.make_desc(2000, 2000, 1984, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
     assert len(G.plan(d)) == 1 and G.plan(d)[0]["variant"] != frag           # edge tiles shifted, K whole
     d = G.make_desc(2000, 2000, 2000, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
-    assert [q["variant"] for q in G.plan(d)] == [frag]                        # K tail: rounding points must not move
+    assert len(G.plan(d)) == 1 and G.plan(d)[0]["variant"] != frag           # K = 64 q + 16: the last slot is shifted back
+    assert G.acc_chunk(d) == 64                                               # ... and rounds after its 16 new k-values
+    for k, tiled in ((48, False), (64, True), (80, True), (4112, True)):
+        d = G.make_desc(512, 512, k)
+        assert (G.plan(d)[0]["variant"] != frag) == tiled and len(G.plan(d)) == 1, k
 
 
 def test_variant_table_and_selection(miw):
@@ -259,19 +263,19 @@ def test_variant_table_and_selection(miw):
                for v in vs[:-1] if not v["pingpong"])
     by = {v["name"]: v["id"] for v in vs}
     # small or odd shapes fall to smaller tiles / fragment ops;
-    # 4096^3 fills 256 CUs with 256x256 tiles: the ping-pong kernel where its rings fit in LDS (at most one
-    # operand with k contiguous), else the kernel with two 64-k slots
+    # 4096^3 fills 256 CUs with 256x256 tiles: the ping-pong kernel, in every operand layout
     W = miw.WMMA
     assert vs[G.pick_variant(G.make_desc(4096, 4096, 4096)) - 1]["name"] == "tile256x256_pingpong"
     rc = G.make_desc(4096, 4096, 4096, a_layout=W.RowMajor, b_layout=W.ColMajor)
-    assert G.pick_variant(rc) == 1 and not G.variant_supports(rc, by["tile256x256_pingpong"])
-    assert G.variant_supports(rc, 1) and not G.variant_supports(G.make_desc(128, 128, 128), 1)
+    assert G.pick_variant(rc) == by["tile256x256_pingpong"]                    # every operand layout has a ring that fits
+    assert not G.variant_supports(G.make_desc(128, 128, 128), by["tile256x256_pingpong"])
     batched = vs[G.pick_variant(G.make_desc(128, 128, 128, batch=512)) - 1]
     assert batched["block"][:2] == (128, 128) and batched["stages"] == 2      # two workgroups per CU
     deep = vs[G.pick_variant(G.make_desc(2048, 2048, 2048)) - 1]
     assert deep["block"][:2] == (128, 128) and deep["stages"] == 4            # one workgroup per CU, long K
     assert G.pick_variant(G.make_desc(48, 48, 48)) == by["fragment_ops"]
-    assert G.pick_variant(G.make_desc(64, 64, 80)) == by["fragment_ops"]
+    assert G.pick_variant(G.make_desc(64, 64, 48)) == by["fragment_ops"]       # less than one slot of K
+    assert G.pick_variant(G.make_desc(64, 64, 80)) == by["tile64x64_w2x2"]     # K = 64 + 16
     # the choice goes by estimated duration, not by tile count alone:
     # 3072^3 is 144 tiles of 256 x 256 (one round on 256 CUs) or 288 of 256 x 128 (two rounds)
     assert vs[G.pick_variant(G.make_desc(3072, 3072, 3072)) - 1]["name"] == "tile256x256_pingpong"
@@ -301,7 +305,7 @@ def test_variant_table_and_selection(miw):
     d = G.make_desc(4096, 4096, 4096, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
     assert vs[G.pick_variant(d) - 1]["f16_accumulate"]
     names = miw.kernel_names()
-    assert "wmma_mac_f32_f32" in names and "gemm_tile256x256_w2x4" in names
+    assert "wmma_mac_f32_f32" in names and "gemm_tile256x128_w4x2" in names
 
 
 def test_no_device_errors_are_clean(miw):
@@ -346,7 +350,7 @@ def test_tiled_gemm_kernels_are_not_launchable_by_name(miw):
     L = miw._lib
     lib = L.load()
     u3 = (ctypes.c_uint * 3)
-    for name in ("gemm_tile256x256_w2x4", "gemm_tile128x128_w2x2", "gemm_tile256x256_pingpong"):
+    for name in ("gemm_tile256x128_w4x2", "gemm_tile128x128_w2x2", "gemm_tile256x256_pingpong"):
         k = ctypes.c_void_p()
         assert lib.miw_kernel_lookup(name.encode(), ctypes.byref(k)) == 0 and k.value
         assert lib.miw_launch(k, u3(1, 1, 1), u3(64, 1, 1), 0, None, None) == L.ERR_UNSUPPORTED
@@ -359,14 +363,16 @@ def test_tile_counts_that_overflow_the_grid_are_refused(miw):
     q = ctypes.c_void_p(4096)
     G = miw.GEMM
     big = 1 << 30
-    for variant in (0, 1, 8, lib.miw_gemm_variant_count()):
+    by = {v["name"]: v["id"] for v in G.variants()}
+    small, large = by["tile64x64_w2x2"], by["tile256x256_pingpong"]
+    for variant in (0, large, small, lib.miw_gemm_variant_count()):
         d = G.make_desc(big, big, 64, variant=variant)
         assert lib.miw_gemm(ctypes.byref(d), q, q, q, q, None) == L.ERR_UNSUPPORTED, variant
-    assert not G.variant_supports(G.make_desc(big, big, 64), 8)
+    assert not G.variant_supports(G.make_desc(big, big, 64), small)
     # a launch holds fewer than 2^32 threads: 2^19 x 2^18 is 2^25 tiles of 64 x 64 with 256 threads each
     # (too many) and 2^21 tiles of 256 x 256 with 512 (fine)
     d = G.make_desc(1 << 19, 1 << 18, 64)
-    assert not G.variant_supports(d, 8) and G.variant_supports(d, 1)
+    assert not G.variant_supports(d, small) and G.variant_supports(d, large)
 
 
 def test_module_entries_check_their_arguments_without_a_device(miw):
@@ -384,3 +390,64 @@ def test_module_entries_check_their_arguments_without_a_device(miw):
     if os.path.exists(path):
         head = open(path, "rb").read(64)
         assert head[:4] == b"\x7fELF" or head.startswith(b"__CLANG_OFFLOAD_BUNDLE__")
+    # headers that describe more than the buffer holds are refused before the loader reads them
+    if os.path.exists(path):
+        image = open(path, "rb").read()
+        for cut in (len(image) // 2, len(image) - 16, 200):
+            assert lib.miw_module_load(image[:cut], cut, ctypes.byref(p)) == L.ERR_INVALID_VALUE and not p.value, cut
+            assert b"truncated" in lib.miw_last_error()
+        # the whole image passes this check (and then needs miw_init, or a device)
+        assert lib.miw_module_load(image, len(image), ctypes.byref(p)) in (L.ERR_NOT_INITIALIZED, 0) or L.last_error()
+
+
+def test_nextwarp_prevwarp(miw):
+    """src/execution.jl:418-426 with the wavefront size of gfx950 (the reference's tests run them with
+    the device's warp size, test/device/execution.jl)."""
+    dev = {"wave_size": 64}
+    assert miw.warpsize(dev) == 64
+    for threads, nxt, prv in ((1, 64, 0), (63, 64, 0), (64, 64, 64), (65, 128, 64), (1000, 1024, 960), (0, 0, 0)):
+        assert miw.nextwarp(dev, threads) == nxt and miw.prevwarp(dev, threads) == prv, threads
+    assert miw.nextwarp({"wave_size": 32}, 33) == 64 and miw.prevwarp({"wave_size": 32}, 33) == 32
+
+
+def test_resolve_sees_what_the_queries_cannot(miw):
+    """miw_gemm_acc_chunk answers for aligned operands with C and D apart; miw_gemm_resolve takes the
+    pointers.  An fp16-accumulate problem whose C is D and whose extents no tile divides runs on the
+    fragment-op kernel (edge tiles may not overlap in place), which rounds every 16 k-values."""
+    G = miw.GEMM
+    d = G.make_desc(272, 272, 256, c_type=np.float16, d_type=np.float16, acc_type=np.float16)
+    base = 1 << 32
+    apart = (base, base + (1 << 24), base + (2 << 24), base + (3 << 24))
+    nfrag = miw._lib.load().miw_gemm_variant_count()
+    assert G.acc_chunk(d) == 64
+    v, chunk = G.resolve(*apart, d)
+    assert chunk == 64 and v == G.pick_variant(d) != nfrag
+    same = (apart[0], apart[1], apart[3], apart[3])
+    v, chunk = G.resolve(*same, d)
+    assert v == nfrag and chunk == 16
+    # operands that are not 16-byte aligned: also the fragment-op kernel
+    odd = (base + 2, apart[1], apart[2], apart[3])
+    assert G.resolve(*odd, d) == (nfrag, 16)
+    # Float32 accumulation: no chunk
+    d32 = G.make_desc(512, 512, 256)
+    assert G.resolve(*apart, d32)[1] == 0
+
+
+def test_static_splitk_chooses_within_its_capacity(miw):
+    """splits = 0 through the static workspace only considers the slice counts whose partial products fit
+    in it, and falls back to one slice (no workspace) rather than failing."""
+    G = miw.GEMM
+    cap = G.splitk_static_capacity()
+    for shape in ((2048, 2048, 16384), (1024, 1024, 8192), (512, 512, 16384), (256, 256, 65536), (4096, 2048, 4096)):
+        d = G.make_desc(*shape)
+        n, nbytes = G.splitk_static_plan(d, 0)
+        free_n, free_bytes = G.splitk_workspace(d, 0)
+        assert nbytes <= cap and nbytes == (0 if n == 1 else n * shape[0] * shape[1] * 4), shape
+        assert n <= free_n or free_bytes > cap, shape
+        if free_bytes <= cap:
+            assert (n, nbytes) == (free_n, free_bytes), shape
+    # a count asked for that does not fit is still refused
+    d = G.make_desc(2048, 2048, 1024)
+    with pytest.raises(miw.MIWError) as e:
+        G.splitk_static_plan(d, 4)
+    assert e.value.code == miw._lib.ERR_UNSUPPORTED

@@ -22,6 +22,24 @@ def test_static_workspace_matches_the_caller_workspace_entry(gpu, orc):
         want = _run_splitk(gpu, orc, g, A, B, C, splits, prefill=2.0, static=False)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), n
         assert orc.normalized_error(g, got, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
+    # nothing is allocated: free device memory is the same before and after the calls.  (One untimed
+    # round first: the HIP runtime itself may grow its kernel-argument pool when a kernel runs for
+    # the first time in a process, whoever launches it.)
+    g = orc.GemmDesc(M=320, N=192, K=2048, a_layout=orc.ROW)
+    A, B, C = _inputs(orc, g, 705)
+    gr = g.resolved()
+    dA, dB, dC = gpu.DeviceArray(A), gpu.DeviceArray(B), gpu.DeviceArray(C)
+    dD = gpu.DeviceArray.undef(np.float32, gr.stride_d)
+    desc = gpu.GEMM.make_desc(g.M, g.N, g.K, a_layout=gpu.WMMA.RowMajor)
+    for splits in (4, 8, 0):
+        gpu.GEMM.gemm_splitk_static(dA, dB, dC, dD, desc, splits=splits)
+    gpu.synchronize()
+    free0 = gpu.mem_info()[0]
+    for splits in (4, 8, 0, 4):
+        gpu.GEMM.gemm_splitk_static(dA, dB, dC, dD, desc, splits=splits)
+        gpu.synchronize()
+        assert gpu.mem_info()[0] == free0, splits
+    assert orc.normalized_error(g, dD.to_host(), orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
     # exact on integers, chosen slice count
     g = orc.GemmDesc(M=256, N=256, K=2048, beta=-1.0)
     A, B, C = _inputs(orc, g, 710, ints=True)
