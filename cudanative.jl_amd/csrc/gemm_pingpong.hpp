@@ -524,27 +524,24 @@ void k_gemm_pp(tiled_params p)
         }
         return c;
     };
+    static_assert(TI % 2 == 0, "the epilogue stores pairs of tiles");
     auto epilogue = [&](bool with_c, bool trans) {
+        auto value = [&](int a, int b) {
+            float4_t v = acc[a][b];
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] *= p.alpha;
+            if (with_c) {
+                float4_t c = read_c(a, b, trans);
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
+            }
+            return v;
+        };
 #pragma unroll
         for (int b = 0; b < TJ; b++)
 #pragma unroll
-            for (int a = 0; a < TI; a++) {
-                float4_t v = acc[a][b];
-#pragma unroll
-                for (int e = 0; e < 4; e++) v[e] *= p.alpha;
-                if (with_c) {
-                    float4_t c = read_c(a, b, trans);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
-                }
-                DT *dst = D + (long)(col + 16 * b) * p.ldd + (row + 16 * a);
-                if constexpr (__is_same(DT, float)) {
-                    *(float4_t *)dst = v;
-                } else {
-                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                    *(half4_t *)dst = h;
-                }
-            }
+            for (int a = 0; a < TI; a += 2)
+                store_tile_pair<DT>(D, p.ldd, i0 + wi * WTI + 16 * a, j0 + wj * WTJ + 16 * b, lane, value(a, b), value(a + 1, b));
     };
     if (!p.use_c || fold_c) epilogue(false, false);
     else if (p.c_trans) epilogue(true, true);
@@ -1008,29 +1005,26 @@ void k_gemm_pp64(tiled_params p)
     MIW_PP_STAMP(4)
 
     // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
+    static_assert(TI % 2 == 0, "the epilogue stores pairs of tiles");
     auto epilogue = [&](bool with_c, bool trans) {
+        auto value = [&](int a, int b) {
+            float4_t v = separate_sum ? cinit[a][b] : acc[a][b];
+            if constexpr (!F16ACC) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] *= p.alpha;
+                if (with_c) {
+                    float4_t c = read_c(a, b, trans);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
+                }
+            }
+            return v;
+        };
 #pragma unroll
         for (int b = 0; b < TJ; b++)
 #pragma unroll
-            for (int a = 0; a < TI; a++) {
-                float4_t v = separate_sum ? cinit[a][b] : acc[a][b];
-                if constexpr (!F16ACC) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] *= p.alpha;
-                    if (with_c) {
-                        float4_t c = read_c(a, b, trans);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
-                    }
-                }
-                DT *dst = D + (long)(col + 16 * b) * p.ldd + (row + 16 * a);
-                if constexpr (__is_same(DT, float)) {
-                    *(float4_t *)dst = v;
-                } else {
-                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                    *(half4_t *)dst = h;
-                }
-            }
+            for (int a = 0; a < TI; a += 2)
+                store_tile_pair<DT>(D, p.ldd, i0 + wi * WTI + 16 * a, j0 + wj * WTJ + 16 * b, lane, value(a, b), value(a + 1, b));
     };
     if (F16ACC || !p.use_c || fold_c) epilogue(false, false);
     else if (p.c_trans) epilogue(true, true);

@@ -249,6 +249,51 @@ __device__ inline void tail_apply(half8_t &f, unsigned keep)
     f = __builtin_bit_cast(half8_t, v);
 }
 
+// Epilogue store of two MFMA tiles that are neighbours along the contiguous dimension of D: tile rows
+// row .. row + 15 (values v0) and row + 16 .. row + 31 (values v1) of the 16 columns col0 .. col0 + 15.
+// In the accumulator layout a lane holds 4 consecutive rows of one column (lane % 16), the four lanes
+// of a column 16 rows: one store instruction would write 16 pieces of 64 bytes (32 for Float16).  Here
+// neighbouring lanes swap one tile's values (a DPP move inside the quad), so that the even columns go
+// out with the first instruction and the odd ones with the second, each column as one piece of 128
+// bytes (64 for Float16): whole cache lines when the tile starts on one.
+__device__ inline unsigned quad_swap(unsigned v)
+{
+    return (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, true);
+}
+template <class DT>
+__device__ inline void store_tile_pair(DT *D, long ldd, int row, int col0, int lane, float4_t v0, float4_t v1)
+{
+    const int r = lane & 15, q = lane >> 4;
+    const bool odd = r & 1;
+    // both instructions: this lane writes rows row + 16 * odd + 4 q .. + 3; column col0 + r - odd, then the next
+    DT *dst = D + (long)(col0 + r - (odd ? 1 : 0)) * ldd + (row + (odd ? 16 : 0) + 4 * q);
+    if constexpr (__is_same(DT, float)) {
+        const uint4_t p = __builtin_bit_cast(uint4_t, v0), t = __builtin_bit_cast(uint4_t, v1);
+        uint4_t s0, s1;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const unsigned ps = quad_swap(p[e]), ts = quad_swap(t[e]);
+            s0[e] = odd ? ts : p[e];   // even column: own upper tile | the even neighbour's lower tile
+            s1[e] = odd ? t[e] : ps;   // odd column: the odd neighbour's upper tile | own lower tile
+        }
+        *(uint4_t *)dst = s0;
+        *(uint4_t *)(dst + ldd) = s1;
+    } else {
+        const half4_t h0 = {(half_t)v0[0], (half_t)v0[1], (half_t)v0[2], (half_t)v0[3]};
+        const half4_t h1 = {(half_t)v1[0], (half_t)v1[1], (half_t)v1[2], (half_t)v1[3]};
+        const uint2_t p = __builtin_bit_cast(uint2_t, h0), t = __builtin_bit_cast(uint2_t, h1);
+        uint2_t s0, s1;
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const unsigned ps = quad_swap(p[e]), ts = quad_swap(t[e]);
+            s0[e] = odd ? ts : p[e];
+            s1[e] = odd ? t[e] : ps;
+        }
+        *(uint2_t *)dst = s0;
+        *(uint2_t *)(dst + ldd) = s1;
+    }
+}
+
 // Ordinal of the direct-to-LDS load issued after MFMA m of a step of nmfma
 // matrix instructions that issues ndma loads, or -1.  The loads are spread
 // evenly over the step: a wavefront's load occupies the texture-address path
@@ -636,29 +681,26 @@ void k_gemm_tiled(tiled_params p)
     }
 
     // Epilogue: each lane owns 4 consecutive i of one column j per MFMA tile.
+    static_assert(TI % 2 == 0, "the epilogue stores pairs of tiles");
     auto epilogue = [&](bool with_c, bool trans) {
+        auto value = [&](int a, int b) {
+            float4_t v = acc[a][b];
+            if constexpr (!F16ACC) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] *= p.alpha;
+                if (with_c) {
+                    float4_t c = read_c(a, b, trans);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
+                }
+            }
+            return v;
+        };
 #pragma unroll
         for (int b = 0; b < TJ; b++)
 #pragma unroll
-            for (int a = 0; a < TI; a++) {
-                float4_t v = acc[a][b];
-                if constexpr (!F16ACC) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] *= p.alpha;
-                    if (with_c) {
-                        float4_t c = read_c(a, b, trans);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] = __builtin_fmaf(p.beta, c[e], v[e]);
-                    }
-                }
-                DT *dst = D + (long)(col + 16 * b) * p.ldd + (row + 16 * a);
-                if constexpr (__is_same(DT, float)) {
-                    *(float4_t *)dst = v;
-                } else {
-                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                    *(half4_t *)dst = h;
-                }
-            }
+            for (int a = 0; a < TI; a += 2)
+                store_tile_pair<DT>(D, p.ldd, i0 + wi * WTI + 16 * a, j0 + wj * WTJ + 16 * b, lane, value(a, b), value(a + 1, b));
     };
     if (F16ACC || !p.use_c || fold_c) epilogue(false, false);
     else if (p.c_trans) epilogue(true, true);
