@@ -247,19 +247,21 @@ void k_gemm_pp(tiled_params p)
         else lds_dma16_at<XB + I * NT * 16, I * 256>(Y, yvo[0], wave_dst + unit);
     };
     // Past the end of K the last unit is requested again, into a unit nobody reads any more.
-    // k-values from one unit to the next; the first unit of the last pair (pair NP - 1, or entry NS - 2)
-    // lies tail_skip short of where it would follow on (a step back for an entry of 32 when 48 repeat).
+    // Elements from one unit to the next; the first unit of the last pair (pair NP - 1, or entry NS - 2)
+    // lies tail_skip k-values short of where it would follow on (a step back for an entry of 32 when 48
+    // repeat).  Both steps are kept as 64-bit values: computed per request, the multiplication by the
+    // leading dimension is a chain of scalar instructions at the end of every memory cluster, which is
+    // the longer of the two clusters.
+    constexpr int XUK = XK ? KGRAN : BKS, YUK = YK ? KGRAN : BKS;
+    const long xunit = XK ? (long)XUK : (long)XUK * p.ldx, xtail = XK ? (long)(XUK - tail_skip) : (long)(XUK - tail_skip) * p.ldx;
+    const long yunit = YK ? (long)YUK : (long)YUK * p.ldy, ytail = YK ? (long)(YUK - tail_skip) : (long)(YUK - tail_skip) * p.ldy;
     auto x_advance = [&]() {
         xnext++;
-        constexpr int UK = XK ? KGRAN : BKS;
-        const int kstep = xnext == (XK ? NP - 1 : NS - 2) ? UK - tail_skip : xnext < (XK ? NP : NS) ? UK : 0;
-        X += XK ? (long)kstep : (long)kstep * p.ldx;
+        X += xnext == (XK ? NP - 1 : NS - 2) ? xtail : xnext < (XK ? NP : NS) ? xunit : 0;
     };
     auto y_advance = [&]() {
         ynext++;
-        constexpr int UK = YK ? KGRAN : BKS;
-        const int kstep = ynext == (YK ? NP - 1 : NS - 2) ? UK - tail_skip : ynext < (YK ? NP : NS) ? UK : 0;
-        Y += YK ? (long)kstep : (long)kstep * p.ldy;
+        Y += ynext == (YK ? NP - 1 : NS - 2) ? ytail : ynext < (YK ? NP : NS) ? yunit : 0;
     };
     // Request number N (0 .. ND-1) of the memory cluster of k-step 2 pr + H: the X loads, then the Y loads.
     auto cluster_request = [&]<int H, int N>(std::integral_constant<int, H>, std::integral_constant<int, N>) {
@@ -368,6 +370,9 @@ void k_gemm_pp(tiled_params p)
         [&]<int... U>(std::integer_sequence<int, U...>) {
             (cluster_unit(xu, yu, h, std::integral_constant<int, U>{}), ...);
         }(std::make_integer_sequence<int, NFRAG>{});
+        // The ring state and the operand pointers move on here, behind the last fragment read and under its
+        // latency.  (Measured: the same scalar instructions between the first MFMAs of the compute cluster
+        // hold the matrix core up for 65 cycles per cluster; between the fragment reads, for 19.)
         cluster_advance(h);
         if constexpr (H == 1) pair_advance();
         __builtin_amdgcn_sched_barrier(0);
@@ -972,7 +977,14 @@ void k_gemm_pp64(tiled_params p)
             for (int a = 0; a < TI; a++)
 #pragma unroll
                 for (int b = 0; b < TJ; b++) acc[a][b] = cinit[a][b];
-            for (int pr = 0; pr < NPM; pr++) pair(no_fold, rolling);
+            for (int pr = 0; pr < NPM; pr++) {
+#ifdef MIW_PP_TS
+                if (pr == NPM / 2) MIW_PP_STAMP(2)
+                if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
+#endif
+                pair(no_fold, rolling);
+            }
+            MIW_PP_STAMP(9)
             pair(last_pair, rolling);
         }
     } else {
