@@ -38,12 +38,7 @@
 
 namespace miw {
 
-// Measurement switch, 0 in every shipped build: bit 0 drops the direct-to-LDS loads of the K loop,
-// bit 1 its fragment reads (the registers keep the prologue's fragments), bit 2 its MFMAs.  The
-// results are wrong; the timings say what each unit costs in cycles and, under the power cap, in clock.
-#ifndef MIW_PP_ABLATE
-#define MIW_PP_ABLATE 0
-#endif
+// (The measurement switch MIW_PP_ABLATE of gemm_tiled.hpp applies to the loops of these kernels too.)
 
 
 // Second measurement switch (off in every shipped build; gemm_kernels.hip must be compiled with it
@@ -687,8 +682,9 @@ void k_gemm_pp64(tiled_params p)
         next++;
         wslot = wslot + 1 == NSLOT ? 0 : wslot + 1;
         const int kstep = next < NP - 1 ? KGRAN : next == NP - 1 ? KGRAN - tail_skip : 0;
-        X += XK ? (long)kstep : (long)kstep * p.ldx;
-        Y += YK ? (long)kstep : (long)kstep * p.ldy;
+        // (64 leading dimensions fit in 32 bits: the host checks that 256 do)
+        X += XK ? kstep : kstep * (int)p.ldx;
+        Y += YK ? kstep : kstep * (int)p.ldy;
     };
 
     // fp16 accumulation: the C operand is requested first, as raw bits that no instruction touches
@@ -846,11 +842,13 @@ void k_gemm_pp64(tiled_params p)
         __builtin_amdgcn_sched_barrier(0);
     };
     // ZERO (fp16 accumulation with alpha != 1): the accumulators restart from zero in every slot.
-    constexpr int ROUND_LAG = 2;
     auto tile_of_mfma = [](int m) { return m / TJ * TJ + serpentine_column(m, TJ); };
+    // (fp16 accumulation, measured: with both k-steps of a tile back to back, so that the tiles finish
+    // one after the other and the conversions spread over the whole cluster, the second MFMA of a tile
+    // waits for the first and the launch takes 6 to 15 % longer.)
+    constexpr int ROUND_LAG = 2;
     auto compute_cluster = [&]<bool ZERO>(std::bool_constant<ZERO>) {
         __builtin_amdgcn_sched_barrier(0);
-
 #pragma unroll
         for (int h = 0; h < 2; h++)
 #pragma unroll

@@ -55,6 +55,13 @@ typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
 #define MIW_LDS __attribute__((address_space(3)))
 #define MIW_GLOBAL __attribute__((address_space(1)))
 
+// Measurement switch, 0 in every shipped build: bit 0 drops the direct-to-LDS loads of the K loop,
+// bit 1 its fragment reads (the registers keep the prologue's fragments), bit 2 its MFMAs.  The
+// results are wrong; the timings say what each unit costs in cycles and, under the power cap, in clock.
+#ifndef MIW_PP_ABLATE
+#define MIW_PP_ABLATE 0
+#endif
+
 constexpr int BKS = 32;    // k-values per pipeline step (one MFMA k-step)
 constexpr int KGRAN = 64;  // k-values per LDS slot and K granularity of the kernel
 
@@ -471,8 +478,9 @@ void k_gemm_tiled(tiled_params p)
         next++;
         wslot = wslot + 1 == NSLOT ? 0 : wslot + 1;
         const int kstep = next < NP - 1 ? KGRAN : next == NP - 1 ? KGRAN - tail_skip : 0;
-        X += XK ? (long)kstep : (long)kstep * p.ldx;
-        Y += YK ? (long)kstep : (long)kstep * p.ldy;
+        // (64 leading dimensions fit in 32 bits: the host checks that 256 do)
+        X += XK ? kstep : kstep * (int)p.ldx;
+        Y += YK ? kstep : kstep * (int)p.ldy;
     };
     auto request_pair = [&]() {
         begin_request();
@@ -527,11 +535,11 @@ void k_gemm_tiled(tiled_params p)
                  // two take turns.
                  if constexpr (NMFMA >= 8 && m == 0) __builtin_amdgcn_s_setprio(1);
                  if constexpr (NMFMA >= 8 && m == NMFMA / 2) __builtin_amdgcn_s_setprio(0);
-                 if constexpr (m < NUNIT) fetch_unit(nxt, xs, std::integral_constant<int, m>{}, h);
+                 if constexpr (m < NUNIT && !(MIW_PP_ABLATE & 2)) fetch_unit(nxt, xs, std::integral_constant<int, m>{}, h);
                  constexpr int a = m / TJ, b = m % TJ;
-                 acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.x[a], cur.y[b], acc[a][b], 0, 0, 0);
+                 if constexpr (!(MIW_PP_ABLATE & 4)) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.x[a], cur.y[b], acc[a][b], 0, 0, 0);
                  constexpr int d = dma_after_mfma(m, NMFMA, NDMA);
-                 if constexpr (d >= 0) {
+                 if constexpr (d >= 0 && !(MIW_PP_ABLATE & 1)) {
                      __builtin_amdgcn_sched_barrier(0);
                      request_one(std::integral_constant<int, DMA_LO + d>{});
                  }
@@ -565,6 +573,7 @@ void k_gemm_tiled(tiled_params p)
     [&]<int... U>(std::integer_sequence<int, U...>) {
         (fetch_unit(f0, lds, std::integral_constant<int, U>{}, first_half), ...);
     }(std::make_integer_sequence<int, NUNIT>{});
+    if constexpr (MIW_PP_ABLATE & 2) f1 = f0;
 
     // Folding C.  With alpha == 1 the C operand is added into the accumulators
     // during the last NCT trips of the loop, CPT MFMA tiles per trip, so that
