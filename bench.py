@@ -395,7 +395,8 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 in, f16 accumulate" if half else "f16 in, f32 accumulate", "data": "synthetic",
         "config": {"workload": cfg["workload"], "variant": vinfo["name"], "batch": batch,
-                   "operand_sets": len(sets), "operand_scale": args.operand_scale, "cold": cold, "library_build_id": build_id,
+                   "operand_sets": len(sets), "operand_scale": args.operand_scale, "spinup_seconds": args.spinup_seconds,
+                   "cold": cold, "library_build_id": build_id,
                    "algorithmic_flop": flops, "algorithmic_bytes": abytes,
                    "normalized_error_sampled": err, "tolerance": 1e-2 if half else 1e-3,
                    "pct_of_fp16_dense_peak": 100.0 * value / PEAK_F16_DENSE_TFLOPS,

@@ -304,9 +304,8 @@ int check_gemm(const miw_gemm_desc *d, const miw::gemm_params &p, bool f16acc, b
     } else if (!tiled_fits(variant - 1, p, d->c_type, d->d_type, f16acc, d->acc_chunk, in_place)) {
         return fail(MIW_ERR_UNSUPPORTED,
                     "gemm: variant %d (%s) needs M and N of at least one tile (whole tiles when C and D share memory), "
-                    "K divisible by 64, 16-byte aligned operands and leading "
-                    "dimensions, a tile count that fits the launch grid, and (ping-pong kernels) at most one operand "
-                    "with k contiguous%s",
+                    "K of at least 64, 16-byte aligned operands and leading "
+                    "dimensions, and a tile count that fits the launch grid%s",
                     variant, miw::tiled_variant_at(variant - 1).name,
                     f16acc ? ", alpha == 1 (the 64-k ping-pong kernels take any alpha), its own acc_chunk, and accumulators that fit in VGPRs" : "");
     }

@@ -66,7 +66,7 @@ int tiled_f16acc_chunk();
 // Variants whose accumulators do not fit in ordinary VGPRs have no fp16-accumulate form.
 bool tiled_supports_f16acc(int i);
 // Launches tiled variant i.  The caller has checked what the kernels assume: M and N of at least
-// one tile (whole tiles when C and D share memory), K a multiple of 64, 16-byte alignment of
+// one tile (whole tiles when C and D share memory), K of at least 64, 16-byte alignment of
 // pointers and leading dimensions, and for fp16 accumulation c_type == d_type == Float16 and,
 // outside the 64-k ping-pong kernels, alpha == 1.
 hipError_t launch_gemm_tiled(int i, const gemm_params &p, int c_type, int d_type, bool f16acc, hipStream_t s);

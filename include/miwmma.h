@@ -207,7 +207,7 @@ typedef struct miw_gemm_variant_info {
 } miw_gemm_variant_info;
 int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
 /* *supported = 1 when `variant` (1..count) can run this descriptor (M and N of at least one tile,
-   K a multiple of 64, leading dimensions, operand layouts, accumulate type; pointers are assumed
+   K of at least 64, leading dimensions, accumulate type; pointers are assumed
    16-byte aligned and C and D apart), else 0. */
 int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *supported);
 /* Variant of a single launch of this descriptor (what miw_gemm runs unless miw_gemm_plan
@@ -217,15 +217,16 @@ int miw_gemm_variant_supports(const miw_gemm_desc *desc, int variant, int *suppo
 int miw_gemm_pick_variant(const miw_gemm_desc *desc, int *variant);
 /* The launches miw_gemm makes for this descriptor (no counterpart in the reference, whose GEMM
    would be the caller's own kernel over docs/src/device/wmma.md:51-52).  The LDS-tiled kernels take any M and N of
-   at least one tile (multiples of 16, as everywhere): where the tile does not divide an extent
-   the last tile is shifted back so that it ends at the edge and overlaps its neighbour; both
-   workgroups compute the overlap from the same operands in the same order and store equal
-   values.  When C and D share memory (in_place != 0 here; miw_gemm looks at the pointers) that is
-   not allowed and only whole tiles are used.  Beyond that, with Float32 accumulation and
-   desc.variant 0, a problem is cut into parts, each a GEMM on a block of D with offset pointers,
-   launched in order on the caller's stream, where the estimate says that is faster:
-     k = 64 q + r (Float32 D only): the first 64 q k-values, then the last r through the
-       fragment-op kernel with D as its C operand (one more Float32 rounding per element);
+   at least one tile and any K of at least 64 (multiples of 16, as everywhere).  Where the tile does
+   not divide an extent the last tile is shifted back so that it ends at the edge and overlaps its
+   neighbour; both workgroups compute the overlap from the same operands in the same order and
+   store equal values.  When C and D share memory (in_place != 0 here; miw_gemm looks at the
+   pointers) that is not allowed and only whole tiles are used.  Where 64 does not divide K the
+   last slot of 64 k-values is shifted back so that it ends at K, and the k-values it repeats are
+   zeroed in the fragments: K is never cut, and with Float16 accumulation the last rounding follows
+   the last K mod 64 k-values.  Beyond that, with Float32 accumulation and desc.variant 0, a problem
+   is cut into parts, each a GEMM on a block of D with offset pointers, launched in order on the
+   caller's stream, where the estimate says that is faster:
      whole large tiles, then a bottom strip and a right strip, each planned again (4160 rows:
        sixteen rows of 256 x 256 tiles and a strip of 64 x 64 tiles rather than seventeen rows of
        large tiles, which would take two rounds over the CUs).
