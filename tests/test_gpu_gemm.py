@@ -709,6 +709,11 @@ def test_f16acc_exact_on_integers_all_variants(gpu, orc):
             continue
         D = _run(gpu, orc, g, A, B, C, variant=v["id"], acc_type=F16)
         assert np.array_equal(D, orc.gemm_f16acc(g, 16, A, B, C)), v["name"]
+        if not v["fragment_ops"]:                         # one slot of K: the only pair is the last pair
+            g1 = orc.GemmDesc(M=M, N=N, K=64, c_type=orc.F16, d_type=orc.F16, alpha=1.0, beta=-1.0)
+            A, B, C = _inputs(orc, g1, 72, ints=True)
+            D = _run(gpu, orc, g1, A, B, C, variant=v["id"], acc_type=F16)
+            assert np.array_equal(D, orc.gemm_f16acc(g1, 64, A, B, C)), v["name"]
 
 
 def test_f16acc_alpha_beta(gpu, orc):
