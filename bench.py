@@ -119,14 +119,16 @@ SWEEP_SHAPES = [(512, 512, 512), (1024, 1024, 1024), (1536, 1536, 1536), (2048, 
                 (4096, 4096, 4112), (2000, 2000, 2000)]
 
 
-def shape_sweep(vendor):
+def shape_sweep(mode):
     """A comparison aid: Float16 operands in U[-1,1), A column-major and row-major with B column-major, over
-    SWEEP_SHAPES.  This library (Float32 C and D, D = A*B + C): the launches miw_gemm makes by itself and, for
+    SWEEP_SHAPES.  'library' (Float32 C and D, D = A*B + C): the launches miw_gemm makes by itself and, for
     a size a tile divides, every single variant that can run it, each after 0.25 s of untimed launches,
-    median of 30 event-timed launches.  vendor: torch.matmul (hipBLASLt / rocBLAS; Float16 out, no C) timed
-    over 30 back-to-back launches.  The two use different HIP runtimes, hence two invocations."""
+    median of 30 event-timed launches.  'library-f16out': miw_gemm's own launches for D = A*B with a Float16
+    D and no C operand, the vendor call's problem.  'vendor': torch.matmul (hipBLASLt / rocBLAS; Float16 out,
+    no C) timed over 30 back-to-back launches.  The library and torch use different HIP runtimes, hence
+    separate invocations."""
     out = []
-    if vendor:
+    if mode == "vendor":
         import torch
         for M, N, K in SWEEP_SHAPES:
             row = {"shape": [M, N, K]}
@@ -161,17 +163,20 @@ def shape_sweep(vendor):
             G.gemm_bench(*bufs, desc, warmup=0, iters=20)
         return float(np.median(G.gemm_bench(*bufs, desc, warmup=5, iters=30))) * 1e3
 
+    f16out = mode == "library-f16out"
+    kind = dict(d_type=W.Float16, use_c=False) if f16out else {}
     for M, N, K in SWEEP_SHAPES:
         bufs = (m.DeviceArray(rng.uniform(-1, 1, M * K).astype(np.float16)), m.DeviceArray(rng.uniform(-1, 1, K * N).astype(np.float16)),
-                m.DeviceArray(rng.uniform(-1, 1, M * N).astype(np.float32)), m.DeviceArray.undef(np.float32, M * N))
+                m.DeviceArray(rng.uniform(-1, 1, M * N).astype(np.float32)),
+                m.DeviceArray.undef(np.float16 if f16out else np.float32, M * N))
         row = {"shape": [M, N, K]}
         for name, la in (("A col-major", W.ColMajor), ("A row-major", W.RowMajor)):
-            desc = G.make_desc(M, N, K, a_layout=la)
+            desc = G.make_desc(M, N, K, a_layout=la, **kind)
             plan = G.plan(desc)
             r = {"us": round(timed(desc, bufs, 0.25), 1),
                  "launches": ["%s %dx%dx%d" % (names[q["variant"]], q["m"], q["n"], q["k"]) for q in plan]}
             best = None
-            for v in G.variants():
+            for v in () if f16out else G.variants():
                 d2 = G.make_desc(M, N, K, a_layout=la, variant=v["id"])
                 if v["fragment_ops"] or not G.variant_supports(d2, v["id"]) or (len(plan) == 1 and plan[0]["variant"] == v["id"]):
                     continue
@@ -183,7 +188,7 @@ def shape_sweep(vendor):
             row[name] = r
         out.append(row)
         del bufs
-    print(json.dumps({"shape_sweep": "miw_gemm, Float32 C and D", "library_build_id": m._lib.load().miw_build_id().decode(), "rows": out}))
+    print(json.dumps({"shape_sweep": "miw_gemm, Float16 D, no C" if f16out else "miw_gemm, Float32 C and D", "library_build_id": m._lib.load().miw_build_id().decode(), "rows": out}))
 
 
 def main():
@@ -203,9 +208,11 @@ def main():
     ap.add_argument("--library-reference", action="store_true",
                     help="instead of this library, time the vendor GEMM (hipBLASLt / rocBLAS through torch.matmul) on "
                          "4096^3 Float16 operands in the four operand layouts and print one line; a comparison aid")
-    ap.add_argument("--shape-sweep", choices=("library", "vendor"),
+    ap.add_argument("--shape-sweep", choices=("library", "library-f16out", "vendor"),
                     help="instead of the benchmark, time a list of shapes (sizes tiles divide, ragged and thin ones): "
-                         "'library' this library's own choice of launches beside every single variant, 'vendor' torch.matmul")
+                         "'library' this library's own choice of launches beside every single variant (Float32 C and D), "
+                         "'library-f16out' its own choice for a Float16 D and no C (the vendor call's problem), "
+                         "'vendor' torch.matmul")
     ap.add_argument("--operand-scale", type=float, default=1.0,
                     help="multiply A and B by this before rounding to Float16 (0: all-zero operands, which lift the "
                          "power cap off the matrix cores; a measurement aid, not the benchmark)")
@@ -227,7 +234,7 @@ def main():
         library_reference()
         return
     if args.shape_sweep:
-        shape_sweep(args.shape_sweep == "vendor")
+        shape_sweep(args.shape_sweep)
         return
     from __graft_entry__ import load_package
     from oracle import oracle as orc

@@ -10,7 +10,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmiwmma.so")
-SOURCES = ["gemm_tile_256x128.hip", "gemm_tile_256x256_w2x2.hip", "gemm_tile_small.hip", "gemm_tile_pp.hip", "gemm_tile_pp64.hip",
+SOURCES = ["gemm_tile_256x128.hip", "gemm_tile_256x256_w2x2.hip", "gemm_tile_small.hip", "gemm_tile_pp.hip", "gemm_tile_pp64.hip", "gemm_tile_wave128.hip",
            "capi.hip", "frag_kernels.hip", "gemm_kernels.hip"]
 
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")

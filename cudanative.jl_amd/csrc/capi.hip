@@ -157,6 +157,7 @@ bool tiled_fits(int i, const miw::gemm_params &p, int c_type, int d_type, bool f
     // In canonical terms bm tiles the contiguous dimension of D.
     const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
     if (I < v.bm || J < v.bn || p.K < v.bk) return false;  // (K is a multiple of 16: a last slot that 64 does not divide is shifted back and masked)
+    if (v.kind == miw::KIND_WAVE128 && p.K < 2 * v.bk) return false;  // (its loop is peeled over the last two slots)
     if ((I % v.bm || J % v.bn) && in_place) return false;
     if (!miw::tiled_supports_layout(i, p) || !miw::tiled_grid_fits(i, p)) return false;
     if (!aligned16(p.A) || !aligned16(p.B) || !aligned16(p.D) || (p.use_c && !aligned16(p.C))) return false;
@@ -256,6 +257,20 @@ double estimate_us(int i, const miw::gemm_params &p, int c_type, int d_type)
     return 4.5 * (double)rounds + cd_bytes / 5.5e6 + (double)((p.K + v.bk - 1) / v.bk) * per_pair;
 }
 
+// The one-wavefront-per-SIMD kernel reads C in its epilogue (its accumulators live in AGPRs, out of the
+// VALU's reach, so C is not folded into the K loop), and a CU never overlaps one workgroup's epilogue
+// with another's loop: measured against the ping-pong kernel of the same tile it is 1 to 5 % ahead on a
+// problem without a C operand whose tiles the CUs take in one round, level on longer ones, and 4 to 24 %
+// behind whenever C is read.
+bool wave128_pays(int i, const miw::gemm_params &p)
+{
+    const miw::tiled_variant &v = miw::tiled_variant_at(i);
+    const int cus = g_cu_count > 0 ? g_cu_count : 256;
+    const long I = p.d_row ? p.N : p.M, J = p.d_row ? p.M : p.N;
+    const long tiles = ((I + v.bm - 1) / v.bm) * ((J + v.bn - 1) / v.bn) * p.batch;
+    return !p.use_c && tiles <= cus;
+}
+
 // Tiled variants from large tiles to small, of two kernels for one tile the ping-pong form first.
 const std::vector<int> &variant_order()
 {
@@ -280,6 +295,7 @@ int pick_variant(const miw::gemm_params &p, int c_type, int d_type, bool f16acc,
     double best_us = 0.0;
     for (int i : order) {
         if (!tiled_fits(i, p, c_type, d_type, f16acc, acc_chunk, in_place)) continue;
+        if (miw::tiled_variant_at(i).kind == miw::KIND_WAVE128 && !wave128_pays(i, p)) continue;
         const double us = estimate_us(i, p, c_type, d_type);
         if (best < 0 || us < 0.97 * best_us) { best = i; best_us = us; }
     }
@@ -394,6 +410,7 @@ struct gemm_planner {
                     if (mb == 0 || nb == 0 || (mb == p.M && nb == p.N)) continue;
                     const miw::gemm_params body = sub_block(p, c_type, d_type, 0, mb, 0, nb);
                     if (!tiled_fits(i, body, c_type, d_type, false, 0, in_place)) continue;
+                    if (v.kind == miw::KIND_WAVE128 && !wave128_pays(i, body)) continue;
                     std::vector<gemm_part> cand;
                     cand.push_back(gemm_part{i + 1, c_type, body, m0, n0, k0});
                     double us = estimate_us(i, body, c_type, d_type);
@@ -777,7 +794,7 @@ int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out)
     out->block_m = v.bm; out->block_n = v.bn; out->block_k = v.bk;
     out->waves_m = v.wm; out->waves_n = v.wn; out->stages = v.stages; out->lds_bytes = v.lds_bytes;
     out->f16_accumulate = miw::tiled_supports_f16acc(variant - 1) ? 1 : 0;
-    out->pingpong = v.kind == miw::KIND_PINGPONG32 || v.kind == miw::KIND_PINGPONG64;
+    out->pingpong = v.kind == miw::KIND_PINGPONG32 || v.kind == miw::KIND_PINGPONG64 ? 1 : v.kind == miw::KIND_WAVE128 ? 2 : 0;
     return 0;
 }
 

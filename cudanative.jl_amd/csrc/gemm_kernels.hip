@@ -25,6 +25,7 @@ static const tiled_variant g_variants[] = {
     {"tile256x128_pingpong", 256, 128, KGRAN, 4, 2, 3, 3 * (256 + 128) * KGRAN * 2, 2, 1, 0.785f, 0.785f},
     {"tile128x256_pingpong", 128, 256, KGRAN, 2, 4, 3, 3 * (128 + 256) * KGRAN * 2, 2, 1, 0.785f, 0.785f},
     {"tile128x128_pingpong", 128, 128, KGRAN, 4, 2, 4, 4 * (128 + 128) * KGRAN * 2, 2, 1, 0.50f, 0.50f},
+    {"tile256x256_wave128", 256, 256, KGRAN, 2, 2, 3, 160 * 1024, KIND_WAVE128, 1, 1.27f, 1.27f},
 };
 
 int tiled_variant_count() { return (int)(sizeof(g_variants) / sizeof(g_variants[0])); }
@@ -33,7 +34,7 @@ int tiled_f16acc_chunk() { return KGRAN; }
 bool tiled_supports_f16acc(int i)
 {
     const tiled_variant &v = g_variants[i];
-    if (v.kind == KIND_PINGPONG32) return false;  // 32-k clusters: fp32 accumulation only
+    if (v.kind == KIND_PINGPONG32 || v.kind == KIND_WAVE128) return false;  // 32-k clusters, accumulators in AGPRs: fp32 accumulation only
     if (v.kind == KIND_PINGPONG64) return true;   // 64-k clusters round in the compute cluster
     return waves_per_simd(v.bm, v.bn, v.wm * v.wn * 64) >= 2;
 }
@@ -48,6 +49,7 @@ const void *tiled_kernel_128x128_w2x2(bool xk, bool yk, int c_type, int d_type, 
 const void *tiled_kernel_64x64_w2x2(bool xk, bool yk, int c_type, int d_type, bool f16acc);
 const void *pp_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type);
 int pp_lds(int bm, int bn, bool xk, bool yk);
+const void *w128_kernel(bool xk, bool yk, int c_type, int d_type);
 const void *pp64_kernel(int bm, int bn, bool xk, bool yk, int c_type, int d_type, bool f16acc);
 
 
@@ -57,6 +59,7 @@ static const void *pick_kernel(int i, bool xk, bool yk, int c_type, int d_type, 
     const tiled_variant &v = g_variants[i];
     if (v.kind == KIND_PINGPONG32) return f16acc ? nullptr : pp_kernel(v.bm, v.bn, xk, yk, c_type, d_type);
     if (v.kind == KIND_PINGPONG64) return pp64_kernel(v.bm, v.bn, xk, yk, c_type, d_type, f16acc);
+    if (v.kind == KIND_WAVE128) return f16acc ? nullptr : w128_kernel(xk, yk, c_type, d_type);
     const int waves = v.wm * v.wn;
     if (v.bm == 256 && v.bn == 256 && waves == 4) return tiled_kernel_256x256_w2x2(xk, yk, c_type, d_type, f16acc);
     if (v.bm == 256 && v.bn == 128) return tiled_kernel_256x128_w4x2(xk, yk, c_type, d_type, f16acc);
@@ -89,6 +92,7 @@ static void canonical_layout(const gemm_params &g, bool *xk, bool *yk)
 
 bool tiled_supports_layout(int i, const gemm_params &g)
 {
+    if (g_variants[i].kind == KIND_WAVE128) return true;  // (the ping-pong kernel's rings: one fits for every layout)
     if (g_variants[i].kind != KIND_PINGPONG32) return true;
     bool xk, yk;
     canonical_layout(g, &xk, &yk);
@@ -151,7 +155,7 @@ hipError_t launch_gemm_tiled(int i, const gemm_params &g, int c_type, int d_type
     if (!fn) return hipErrorInvalidValue;
     // (the 64-k ping-pong kernels stage a Float16 C tile beside the ring where both fit)
     const int c_stage = v.kind == KIND_PINGPONG64 && f16acc && v.lds_bytes + v.bm * v.bn * 2 <= 160 * 1024 ? v.bm * v.bn * 2 : 0;
-    const int lds_bytes = v.kind == KIND_PINGPONG32 ? pp_lds(v.bm, v.bn, xk, yk)
+    const int lds_bytes = v.kind == KIND_PINGPONG32 || v.kind == KIND_WAVE128 ? pp_lds(v.bm, v.bn, xk, yk)
                           : v.kind != KIND_PIPELINED ? v.lds_bytes + c_stage
                                                      : v.lds_bytes + fold_stage_bytes(v.bm, v.bn, v.wm * v.wn * 64, v.stages);
     hipError_t e = allow_dynamic_lds(fn, lds_bytes);

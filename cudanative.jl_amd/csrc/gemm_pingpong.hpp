@@ -81,7 +81,7 @@ struct pp_operand {
     static constexpr int UNITS = KMAJOR ? KSLOTS : PP_IMAJOR_ENTRIES;
     static constexpr int BYTES = UNITS * UNIT_BYTES;
     static_assert(NL >= 1 && (!KMAJOR || NL % 2 == 0), "operand must divide over the workgroup");
-    static_assert(NT == 512, "lane offsets below assume 512 threads");
+    static_assert(NT == 512 || NT == 256, "lane offsets below assume 256 or 512 threads");
 
     __device__ static inline unsigned lane_offset(int tid, int ld)
     {

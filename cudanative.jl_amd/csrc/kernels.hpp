@@ -46,7 +46,8 @@ const char *frag_kernel_name(int i);
 enum {
     KIND_PIPELINED = 0,   // gemm_tiled.hpp: every wavefront overlaps its own loads, LDS reads and MFMAs
     KIND_PINGPONG32 = 1,  // gemm_pingpong.hpp: the two wavefronts of a SIMD alternate between MFMA and memory clusters of 32 k-values
-    KIND_PINGPONG64 = 2   // the same with clusters of 64 k-values
+    KIND_PINGPONG64 = 2,  // the same with clusters of 64 k-values
+    KIND_WAVE128 = 3      // gemm_wave128.hpp: one wavefront per SIMD with a 128x128 sub-tile, memory instructions between its MFMAs
 };
 struct tiled_variant {
     const char *name;

@@ -102,7 +102,7 @@ def variants():
         _lib.check(lib.miw_gemm_variant_info_get(v, ctypes.byref(info)))
         out.append({"id": v, "name": info.name.decode(), "block": (info.block_m, info.block_n, info.block_k),
                     "waves": (info.waves_m, info.waves_n), "stages": info.stages, "lds_bytes": info.lds_bytes,
-                    "fragment_ops": bool(info.fragment_ops), "f16_accumulate": bool(info.f16_accumulate), "pingpong": bool(info.pingpong)})
+                    "fragment_ops": bool(info.fragment_ops), "f16_accumulate": bool(info.f16_accumulate), "pingpong": info.pingpong == 1, "wave128": info.pingpong == 2})
     return out
 
 

@@ -686,7 +686,7 @@ function gemm_variants()
         i = info[]
         push!(out, (id=Int(v), name=cstring(i.name), block=(Int(i.block_m), Int(i.block_n), Int(i.block_k)),
                     waves=(Int(i.waves_m), Int(i.waves_n)), stages=Int(i.stages), lds_bytes=Int(i.lds_bytes),
-                    fragment_ops=i.fragment_ops != 0, f16_accumulate=i.f16_accumulate != 0, pingpong=i.pingpong != 0))
+                    fragment_ops=i.fragment_ops != 0, f16_accumulate=i.f16_accumulate != 0, pingpong=i.pingpong == 1, wave128=i.pingpong == 2))
     end
     return out
 end

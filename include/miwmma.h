@@ -203,7 +203,9 @@ typedef struct miw_gemm_variant_info {
     int fragment_ops;   /* 1: built from load_a/load_b/mma on global memory, no LDS */
     int f16_accumulate; /* 1: has a Float16-accumulate form (accumulators fit in ordinary VGPRs) */
     int pingpong;       /* 1: the two wavefronts of a SIMD alternate between matrix-core and memory phases;
-                           lds_bytes is then the largest ring over the operand layouts */
+                           2: one wavefront per SIMD with a 128x128 sub-tile issues its memory instructions
+                           between its MFMAs (K of at least 128); either way lds_bytes is the largest ring
+                           over the operand layouts */
 } miw_gemm_variant_info;
 int miw_gemm_variant_info_get(int variant, miw_gemm_variant_info *out);
 /* *supported = 1 when `variant` (1..count) can run this descriptor (M and N of at least one tile,

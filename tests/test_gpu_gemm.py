@@ -74,7 +74,7 @@ def _vid(gpu, name):
 def _restricted(v):
     """Variants that serve only part of the problem space (operand layouts, K extent): _run checks that
     the library refuses the rest and returns None."""
-    return v["pingpong"]
+    return v["pingpong"] or v["wave128"]
 
 
 def _tile_multiple(v, mult=(1, 1, 2)):
@@ -396,6 +396,9 @@ def test_k_tail_every_variant(gpu, orc, al, bl, dl):
             g = orc.GemmDesc(M=big, N=2 * big if K < 1024 else big, K=K, a_layout=al, b_layout=bl, c_layout=dl, d_layout=dl, beta=-1.0)
             A, B, C = _inputs(orc, g, 1500 + K + v["id"], ints=True)
             D = _run(gpu, orc, g, A, B, C, variant=v["id"])
+            if v["wave128"] and K < 128:
+                assert D is None        # (refused, as _run has checked: its loop is peeled over the last two slots)
+                continue
             assert D is not None and np.array_equal(D, orc.gemm(g, A, B, C)), (v["name"], al, bl, dl, K)
         if not v["f16_accumulate"]:
             continue
@@ -931,3 +934,36 @@ def test_gemm_on_a_created_stream(gpu, orc):
         s.synchronize()
         assert orc.normalized_error(g, dD.to_host(), ref) <= TIGHT_F32
         del ws
+
+
+@pytest.mark.parametrize("al,bl", itertools.product((0, 1), repeat=2))
+def test_wave128_kernel_forced(gpu, orc, al, bl):
+    """The 256x256 kernel with one wavefront per SIMD (accumulators in AGPRs, C added in the epilogue),
+    forced through desc.variant in every operand layout: both D layouts, a C of the other layout, the
+    four C / D type pairs, scalars, batches, padded leading dimensions, extents that 256 does not divide,
+    K with and without a tail, no C operand.  Bit-exact on integers."""
+    v = _vid(gpu, "tile256x256_wave128")
+    F16c, F32c = orc.F16, orc.F32
+    cases = [  # M, N, K, dl, cl, ct, dt, alpha, beta, use_c, batch, pad
+        (256, 256, 128, 0, 0, F32c, F32c, 1.0, 1.0, 1, 1, 0),
+        (512, 256, 208, 1, 1, F16c, F32c, -2.0, 0.5, 1, 2, 8),
+        (272, 528, 320, 0, 1, F32c, F16c, 1.0, -1.0, 1, 1, 16),
+        (768, 512, 368, 1, 0, F16c, F16c, 0.5, 2.0, 1, 1, 0),
+        (512, 512, 256, 0, 0, F32c, F32c, 1.0, 0.0, 0, 3, 0),
+        (256, 512, 1104, 0, 0, F32c, F32c, 1.0, 1.0, 1, 1, 0),
+    ]
+    for n, (M, N, K, dl, cl, ct, dt, alpha, beta, use_c, batch, pad) in enumerate(cases):
+        g0 = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=ct, d_type=dt).resolved()
+        g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=ct, d_type=dt, alpha=alpha,
+                         beta=beta, use_c=use_c, batch=batch, lda=g0.lda + pad, ldb=g0.ldb + pad, ldc=g0.ldc + pad, ldd=g0.ldd + pad)
+        A, B, C = _inputs(orc, g, 2300 + n, ints=True)
+        D = _run(gpu, orc, g, A, B, C if use_c else None, variant=v, prefill=3.0)
+        assert D is not None, (n, al, bl)
+        want = orc.gemm(g, A, B, C)
+        gr = g.resolved()
+        # the padding between columns (rows) of D keeps the prefill
+        other, inner, ld = (M, N, gr.ldd) if dl == orc.ROW else (N, M, gr.ldd)
+        got = D.reshape(batch, -1)[:, :other * ld].reshape(batch, other, ld)
+        ref = want.reshape(batch, -1)[:, :other * ld].reshape(batch, other, ld)
+        assert np.array_equal(got[:, :, :inner], ref[:, :, :inner]), (n, al, bl)
+        assert np.all(got[:, :, inner:] == 3.0), (n, al, bl)

@@ -260,7 +260,7 @@ def test_variant_table_and_selection(miw):
     assert vs[-1]["fragment_ops"] and vs[-1]["name"] == "fragment_ops"
     assert all(v["lds_bytes"] <= 160 * 1024 for v in vs)
     assert all(v["lds_bytes"] == v["stages"] * (v["block"][0] + v["block"][1]) * v["block"][2] * 2
-               for v in vs[:-1] if not v["pingpong"])
+               for v in vs[:-1] if not (v["pingpong"] or v["wave128"]))
     by = {v["name"]: v["id"] for v in vs}
     # small or odd shapes fall to smaller tiles / fragment ops;
     # 4096^3 fills 256 CUs with 256x256 tiles: the ping-pong kernel, in every operand layout
@@ -269,6 +269,14 @@ def test_variant_table_and_selection(miw):
     rc = G.make_desc(4096, 4096, 4096, a_layout=W.RowMajor, b_layout=W.ColMajor)
     assert G.pick_variant(rc) == by["tile256x256_pingpong"]                    # every operand layout has a ring that fits
     assert not G.variant_supports(G.make_desc(128, 128, 128), by["tile256x256_pingpong"])
+    # the one-wavefront-per-SIMD kernel of the same tile: picked where it pays (no C operand to read in its
+    # epilogue, and no more tiles than CUs), never below K = 128
+    assert vs[G.pick_variant(G.make_desc(4096, 4096, 4096, use_c=False)) - 1]["name"] == "tile256x256_wave128"
+    assert vs[G.pick_variant(G.make_desc(4096, 4096, 4096, use_c=False, d_type=np.float16, a_layout=W.RowMajor)) - 1]["wave128"]
+    assert vs[G.pick_variant(G.make_desc(8192, 8192, 1024, use_c=False)) - 1]["name"] == "tile256x256_pingpong"
+    assert G.variant_supports(G.make_desc(512, 512, 128), by["tile256x256_wave128"])
+    assert not G.variant_supports(G.make_desc(512, 512, 112), by["tile256x256_wave128"])
+    assert not G.variant_supports(G.make_desc(512, 512, 256, acc_type=np.float16, c_type=np.float16, d_type=np.float16), by["tile256x256_wave128"])
     batched = vs[G.pick_variant(G.make_desc(128, 128, 128, batch=512)) - 1]
     assert batched["block"][:2] == (128, 128) and batched["stages"] == 2      # two workgroups per CU
     deep = vs[G.pick_variant(G.make_desc(2048, 2048, 2048)) - 1]

@@ -83,3 +83,79 @@ def test_tiled_kernels_keep_spills_out_of_the_steady_state(miw):
         if "256, 256, 2, 2, 2" in name:
             continue    # 256 accumulators per lane: the 4-wavefront tile spills around its loop
         assert sum(1 for l in lines[mfma[0]:mfma[-1]] if re.match(r"\s*scratch_", l)) <= 48, name
+
+
+def _regs(tok):
+    """Registers named by one operand: 'v12' -> {('v', 12)}, 'a[4:7]' -> {('a', 4) .. ('a', 7)}."""
+    m = re.fullmatch(r"([va])(\d+)", tok)
+    if m:
+        return {(m.group(1), int(m.group(2)))}
+    m = re.fullmatch(r"([va])\[(\d+):(\d+)\]", tok)
+    if m:
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    return set()
+
+
+def test_wave128_kernels_keep_the_matrix_instruction_hazards(miw):
+    """The one-wavefront-per-SIMD GEMM kernel writes its MFMAs as inline assembly (accumulators in
+    AGPRs), so the compiler does not keep the distances the hardware asks for around them.  Checked
+    here on the built code of every instance: no MFMA reads a register that a VALU instruction
+    (a copy the register allocator placed, an address addition) wrote less than two wait states
+    before it; no accumulator is copied out of its AGPR less than 18 wait states behind the MFMA
+    that wrote it; the rolled K loops hold neither such copies nor scratch traffic; the accumulators
+    fill the AGPRs and the kernel runs one wavefront per SIMD."""
+    isa = miw.reflection.code_gcn("k_gemm_w128<")
+    assert len(isa) == 16                                       # four layouts x C type x D type
+    res = miw.reflection.kernel_resources()
+    for name, text in isa.items():
+        lines = [l.split("//")[0].strip() for l in text.splitlines()]
+        lines = [l for l in lines if l and not l.startswith(("<", ";"))]
+        ops = [l.replace(",", " ").split() for l in lines]
+        mfma = [i for i, o in enumerate(ops) if o[0].startswith("v_mfma")]
+        assert len(mfma) >= 7 * 64, name                        # the unrolled steps of 8 x 8 tiles
+        for i in mfma:
+            assert ops[i][1].startswith("a[") and ops[i][4] == ops[i][1], (name, lines[i])
+            sources = _regs(ops[i][2]) | _regs(ops[i][3]) | _regs(ops[i][4])
+            wait, j = 0, i - 1
+            while wait < 2 and j >= 0:
+                o = ops[j]
+                if o[0] == "s_nop":
+                    wait += int(o[1]) + 1
+                else:
+                    if o[0].startswith("v_") and not o[0].startswith("v_mfma"):
+                        assert not (_regs(o[1]) & sources), (name, lines[j], lines[i])
+                    assert not o[0].startswith(("s_cbranch", "s_branch", "s_endpgm")), (name, lines[j], lines[i])
+                    wait += 1
+                j -= 1
+        for i, o in enumerate(ops):
+            if o[0] in ("v_accvgpr_read_b32", "v_accvgpr_mov_b32"):
+                src = _regs(o[2])
+                wait, j = 0, i - 1
+                while wait < 18 and j >= 0:
+                    p = ops[j]
+                    if p[0] in ("s_branch", "s_endpgm", "s_setpc_b64"):
+                        break                                   # no fall-through: what precedes in the listing does not run before
+                    if p[0] == "s_nop":
+                        wait += int(p[1]) + 1
+                    else:
+                        assert not (p[0].startswith("v_mfma") and _regs(p[1]) & src), (name, lines[j], lines[i])
+                        wait += 1
+                    j -= 1
+        # the rolled loops: from the target of every backward branch to the branch
+        back = [i for i, o in enumerate(ops) if re.match(r"s_c?branch", o[0]) and o[1].isdigit() and int(o[1]) >= 0x8000]
+        k_loops = 0
+        for b in back:
+            body, words = [], 65536 - int(ops[b][1]) - 1
+            j = b - 1
+            while words > 0 and j >= 0:                         # (MFMAs, loads and reads are two words, most scalar instructions one)
+                body.append(ops[j][0])
+                words -= 1 if ops[j][0].startswith(("s_", "v_add", "v_mov", "v_and")) and "0x" not in lines[j] else 2
+                j -= 1
+            if not any(o.startswith("v_mfma") for o in body):
+                continue                                        # (a loop of the epilogue)
+            k_loops += 1
+            assert sum(o.startswith("v_mfma") for o in body) >= 96, (name, len(body))
+            assert not [o for o in body if o.startswith(("scratch_", "v_accvgpr"))], name
+        assert k_loops == 2, name                               # the loop with the short pointer bookkeeping and the general one
+        (r,) = [v for k, v in res.items() if name in k]
+        assert r["agpr"] == 256 and r["max_threads"] == 256, name
