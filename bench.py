@@ -81,9 +81,10 @@ def cpu_baseline(orc, M, N, K, batch, budget_s=20.0):
     }
 
 
-def library_reference():
+def library_reference(only=None, steps=200, spin=0.3):
     """torch.matmul on 4096^3 Float16 matrices (Float16 output, no C operand; torch.addmm for a Float16 C),
-    timed like the benchmark: spin-up, then 200 back-to-back launches between two synchronisations."""
+    timed like the benchmark: spin-up, then `steps` back-to-back launches between two synchronisations.
+    only: (A layout, B layout) to time that case alone (for a counter run on the vendor's kernel)."""
     import torch
     n = 4096
     a = (torch.rand(n, n, device="cuda") * 2 - 1).half()
@@ -95,18 +96,21 @@ def library_reference():
              "A col-major, B row-major": lambda: torch.matmul(a.t(), b),
              "A row-major, B row-major": lambda: torch.matmul(a, b),
              "A row-major, B row-major, + Float16 C (addmm)": lambda: torch.addmm(c, a, b)}
+    if only:
+        key = "A %s-major, B %s-major" % only
+        cases = {key: cases[key]}
     out = {}
     for name, fn in cases.items():
         t_spin = time.perf_counter()
-        while time.perf_counter() - t_spin < 0.3:
+        while time.perf_counter() - t_spin < spin:
             for _ in range(50):
                 fn()
             torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(200):
+        for _ in range(steps):
             fn()
         torch.cuda.synchronize()
-        t = (time.perf_counter() - t0) / 200
+        t = (time.perf_counter() - t0) / steps
         out[name] = {"us": t * 1e6, "tflops": 2.0 * n ** 3 / t / 1e12}
     print(json.dumps({"library_reference": "torch.matmul Float16 4096^3 (torch %s)" % torch.__version__, "results": out}))
 
@@ -219,6 +223,10 @@ def main():
     ap.add_argument("--skip-check", action="store_true",
                     help="do not fail on a result outside tolerance (measurement builds with parts of the kernel compiled out)")
     ap.add_argument("--no-cold", action="store_true", help="skip the second timed region over four operand sets")
+    ap.add_argument("--no-c", action="store_true",
+                    help="drop the C operand (D = A*B); with --d-type f16 the problem of the vendor call that "
+                         "--library-reference times.  A comparison aid, not the benchmark")
+    ap.add_argument("--d-type", choices=("f32", "f16"), help="override the type of D (Float32 accumulation configurations only)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only run the matrix-core power probe (zero and random operands) and print its line")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -231,7 +239,10 @@ def main():
         sys.exit(2)
 
     if args.library_reference:
-        library_reference()
+        if args.a_layout and args.b_layout:
+            library_reference((args.a_layout[:3], args.b_layout[:3]), args.steps, args.spinup_seconds)
+        else:
+            library_reference()
         return
     if args.shape_sweep:
         shape_sweep(args.shape_sweep)
@@ -266,6 +277,9 @@ def main():
     M, N, K, batch = cfg["M"], cfg["N"], cfg["K"], cfg["batch"]
     half = cfg["half"]
     ct = np.float16 if half else np.float32
+    dt = ct if half or not args.d_type else {"f32": np.float32, "f16": np.float16}[args.d_type]
+    if args.no_c or dt != ct:
+        cfg["workload"] += " [%sFloat%d D]" % ("no C operand, " if args.no_c else "", 8 * np.dtype(dt).itemsize)
     lay = {"col": W.ColMajor, "row": W.RowMajor}
 
     lo, hi, clo, chi = (-0.5, 0.5, -0.1, 0.1) if half else (-1.0, 1.0, -1.0, 1.0)
@@ -281,9 +295,11 @@ def main():
         A = (A.astype(np.float32) * args.operand_scale).astype(np.float16)
         B = (B.astype(np.float32) * args.operand_scale).astype(np.float16)
     dA, dB, dC = m.DeviceArray(A), m.DeviceArray(B), m.DeviceArray(C)
-    dD = m.DeviceArray.undef(ct, batch * M * N)
-    desc = G.make_desc(M, N, K, a_layout=lay[cfg["a"]], b_layout=lay[cfg["b"]], c_type=ct, d_type=ct,
-                       acc_type=ct, batch=batch, variant=args.variant)
+    if args.no_c:
+        C = np.zeros_like(C)     # (what the check below compares with)
+    dD = m.DeviceArray.undef(dt, batch * M * N)
+    desc = G.make_desc(M, N, K, a_layout=lay[cfg["a"]], b_layout=lay[cfg["b"]], c_type=ct, d_type=dt,
+                       acc_type=ct, batch=batch, variant=args.variant, use_c=not args.no_c)
     variant = args.variant or G.pick_variant(desc)
     vinfo = G.variants()[variant - 1]
 
@@ -320,7 +336,7 @@ def main():
     # set smaller than the 256 MiB Infinity Cache is not served from it ("hot" is the default)
     sets = [(dA, dB, dC, dD)]
     for _ in range(1, max(args.rotate, 1)):
-        sets.append((m.DeviceArray(A), m.DeviceArray(B), m.DeviceArray(C), m.DeviceArray.undef(ct, batch * M * N)))
+        sets.append((m.DeviceArray(A), m.DeviceArray(B), m.DeviceArray(C), m.DeviceArray.undef(dt, batch * M * N)))
     wall, ev_ms = timed_region(sets, args.warmup, args.steps)
     # outside the timed region: the same launches again, each bracketed by its own pair of events
     ms = G.gemm_bench(dA, dB, dC, dD, desc, warmup=0, iters=min(args.steps, 50))
@@ -328,7 +344,7 @@ def main():
     # each launch finds its inputs in HBM only
     cold = None
     if len(sets) == 1 and not args.no_cold:
-        cold_sets = sets + [(m.DeviceArray(A), m.DeviceArray(B), m.DeviceArray(C), m.DeviceArray.undef(ct, batch * M * N))
+        cold_sets = sets + [(m.DeviceArray(A), m.DeviceArray(B), m.DeviceArray(C), m.DeviceArray.undef(dt, batch * M * N))
                             for _ in range(3)]
         cwall, cev = timed_region(cold_sets, min(args.warmup, 40), args.steps)
         cold = {"operand_sets": 4, "ms_per_step": cwall * 1e3 / args.steps, "kernel_ms_mean": cev / args.steps,
@@ -354,7 +370,7 @@ def main():
 
     flops = 2.0 * M * N * K * batch
     gdesc = orc.GemmDesc(M=M, N=N, K=K, batch=batch, c_type=orc.F16 if half else orc.F32,
-                         d_type=orc.F16 if half else orc.F32)
+                         d_type=orc.F16 if dt == np.float16 else orc.F32, use_c=0 if args.no_c else 1)
     abytes = gdesc.algorithmic_bytes()
     ms_per_step = wall * 1e3 / args.steps
     value = flops / (wall / args.steps) / 1e12
@@ -376,6 +392,7 @@ def main():
                 "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     family = ("k_gemm_fragops" if vinfo["fragment_ops"] else
+              "k_gemm_w128" if vinfo["wave128"] else
               "k_gemm_tiled" if not vinfo["pingpong"] else
               "k_gemm_pp" if vinfo["block"][:2] == (256, 256) else "k_gemm_pp64")
     roof["kernel"] = "%s<%s>" % (family, vinfo["name"])

@@ -26,10 +26,15 @@
 // loads it issued two steps ago and earlier, and the barrier publishes them: a load has two k-steps
 // (about 2100 cycles) to land.
 //
-// C is added in the epilogue: the VALU cannot reach the AGPRs, so the ping-pong kernels' way of
-// folding C into the last k-steps (loads into registers, fused multiply-adds onto the accumulators)
-// is not open to this kernel, and a problem that reads C pays for it behind the loop (measured on
-// 4096^3: 116.9 us against 107.1 for the ping-pong kernel; without a C operand 104.2 against 105.5).
+// C is added in the epilogue.  The ping-pong kernels fold C into the last k-steps (loads into registers,
+// fused multiply-adds onto the accumulators, under the MFMAs of the other wavefront); here the VALU
+// cannot reach the AGPRs, and an MFMA takes its C operand from the register file it writes its result
+// to (one bit selects AGPRs for both), so a tile cannot pass through ordinary registers on its way
+// from one MFMA to the next: folding would take twelve VALU instructions per tile (four reads, four
+// multiply-adds, four writes) out of issue slots that a lone wavefront needs for its MFMAs.  A problem
+// that reads C therefore pays for it behind the loop (measured on 4096^3: 116.9 us against 107.1 for
+// the ping-pong kernel; without a C operand 104.2 against 105.5), and miw_gemm picks this kernel by
+// itself only for problems without one.
 //
 // The MFMAs are opaque to the compiler, so the hazards between them and other instructions are kept
 // by construction and checked on the built code (tests/test_reflection.py): two MFMAs on one
