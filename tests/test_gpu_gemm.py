@@ -967,3 +967,19 @@ def test_wave128_kernel_forced(gpu, orc, al, bl):
         ref = want.reshape(batch, -1)[:, :other * ld].reshape(batch, other, ld)
         assert np.array_equal(got[:, :, :inner], ref[:, :, :inner]), (n, al, bl)
         assert np.all(got[:, :, inner:] == 3.0), (n, al, bl)
+
+
+@pytest.mark.parametrize("al,bl", itertools.product((0, 1), repeat=2))
+def test_wave128_kernel_bits_equal_the_pingpong_kernel(gpu, orc, al, bl):
+    """Both 256x256 kernels add the k-steps in the same order into Float32 accumulators and apply the
+    scalars the same way behind the loop (K short enough that the ping-pong kernel does not fold C into
+    it): on seeded random operands their results are equal bit for bit, and within tolerance of float64."""
+    w, pp = _vid(gpu, "tile256x256_wave128"), _vid(gpu, "tile256x256_pingpong")
+    for n, (M, N, K, use_c, alpha, beta) in enumerate([(512, 768, 400, 1, 1.0, 1.0), (768, 256, 1008, 1, -0.5, 2.0), (512, 512, 2064, 0, 1.0, 0.0)]):
+        g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, alpha=alpha, beta=beta, use_c=use_c)
+        A, B, C = _inputs(orc, g, 2400 + n)
+        got = _run(gpu, orc, g, A, B, C if use_c else None, variant=w)
+        ref = _run(gpu, orc, g, A, B, C if use_c else None, variant=pp)
+        assert got is not None and ref is not None
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), (n, al, bl)
+        assert orc.normalized_error(g, got, orc.gemm_f64(g, A, B, C)) <= TIGHT_F32
