@@ -50,8 +50,11 @@ namespace miw {
 // MIW_TS holds (cudanative.jl_amd/timestamps.py sets it and prints the phases).
 #ifdef MIW_PP_TS
 #define MIW_PP_STAMP(i) { __builtin_amdgcn_sched_barrier(0); ts[i] = clock64(); __builtin_amdgcn_sched_barrier(0); }
+// (in the unrolled part of the loop: the ring of pairs that holds pair NPM / 2 stamps its first pair)
+#define MIW_PP_MIDDLE(pr) { stamp_pair = (pr) <= NPM / 2 && NPM / 2 < (pr) + NSLOT; if (stamp_pair) MIW_PP_STAMP(2) }
 #else
 #define MIW_PP_STAMP(i)
+#define MIW_PP_MIDDLE(pr)
 #endif
 
 constexpr int PP_KMAJOR_SLOTS = 3;
@@ -566,13 +569,21 @@ void k_gemm_pp(tiled_params p)
 // two barriers that follow publish it before anyone reads it.  Both operand kinds use the slot
 // layouts, loaders and fragment readers of gemm_tiled.hpp.
 //
+// A wavefront issues one instruction in four to five cycles, whatever the instruction, and only one
+// instruction rides for nothing behind each MFMA.  So both clusters are as long as their instruction
+// counts: the memory cluster is kept to the fragment reads, three instructions per load and a handful
+// of scalar ones (the part of the loop that needs no look at the end of K is unrolled over the ring,
+// so that slots are compile-time offsets, and advances the operand origins behind MFMAs of the compute
+// cluster), and the compute cluster to the MFMAs and what must follow them.
+//
 // fp16 accumulation rounds once per slot (64 k-values), two MFMAs after a tile's last MFMA of the pair,
-// inside the compute cluster: at these tiles the memory cluster is the longer of the two (it is bound
-// by the LDS: measured, the same conversions placed between the fragment reads of the next memory
-// cluster cost 15 to 25 % of the launch).  With alpha == 1 the accumulators start as half(beta * C) and
-// the MFMAs accumulate onto the rounded sum in place, otherwise the running sum is kept beside
-// accumulators that restart from zero in every slot: run = half(run + alpha * slot sum).  C is
-// requested before anything else and converted once the first pair's loads have landed.
+// inside the compute cluster, except the cluster's last two tiles, which the wavefront rounds at the
+// end of its next memory cluster (more there, or the conversions between the fragment reads, lengthen
+// the memory cluster beyond the compute cluster: measured, up to 25 % of the launch).  With alpha == 1
+// the accumulators start as half(beta * C) and the MFMAs accumulate onto the rounded sum in place,
+// otherwise the running sum is kept beside accumulators that restart from zero in every slot:
+// run = half(run + alpha * slot sum).  C is requested before anything else and converted once the
+// first pair's loads have landed.
 template <int BI, int BJ, int WI, int WJ, int NSLOT, bool XK, bool YK, class CT, class DT, bool F16ACC>
 __global__ __launch_bounds__(WI *WJ * 64) __attribute__((amdgpu_waves_per_eu(2)))
 void k_gemm_pp64(tiled_params p)
@@ -668,23 +679,47 @@ void k_gemm_pp64(tiled_params p)
     const int tail_skip = NP * KGRAN - p.K;
     const unsigned wave_dst = (unsigned)(uintptr_t)lds + (unsigned)wave * 1024u;
     int next = 0;          // next pair to request
-    int wslot = 0;         // the slot it goes to
+    unsigned woff = 0;     // byte offset in the ring of the slot it goes to
     unsigned dma_dst = 0;  // this wavefront's first destination byte in that slot
-    auto begin_request = [&]() { dma_dst = wave_dst + (unsigned)(wslot * SLOT); };
+    // A wavefront issues little more than one instruction in four to five cycles, whatever the
+    // instruction, and its memory cluster is a chain of some sixty of them: every scalar instruction
+    // spent on addresses there lengthens the cluster as much as a fragment read does.  So a load is
+    // three instructions (M0 written by the addition that forms the LDS address; the global address is
+    // the slot's uniform origin plus a lane offset, the loads of a K-major operand, whose origins lie
+    // a multiple of the leading dimension apart, each with a lane offset of their own, the others with
+    // the instruction's offset field), the ring positions are kept as byte offsets, and the pairs whose
+    // request needs no look at the end of K (FAST) advance the origins by a loop-invariant step.
+    unsigned xvo[XK ? NLX : 1], yvo[YK ? NLY : 1];
+#pragma unroll
+    for (int i = 0; i < (XK ? NLX : 1); i++) xvo[i] = xoff + 2u * (unsigned)xload::load_delta(i, p.ldx);
+#pragma unroll
+    for (int i = 0; i < (YK ? NLY : 1); i++) yvo[i] = yoff + 2u * (unsigned)yload::load_delta(i, p.ldy);
+    auto begin_request = [&]() { dma_dst = wave_dst + woff; };
+    // the same for a pair that reads slot SL, known at compile time: its request goes to the slot before
+    auto begin_request_at = [&]<int SL>(std::integral_constant<int, SL>) { dma_dst = wave_dst + (unsigned)((SL + NSLOT - 1) % NSLOT * SLOT); };
     auto request_one = [&]<int I>(std::integral_constant<int, I>) {
-        if constexpr (I < NLX)
-            lds_dma16(X + xload::load_delta(I, p.ldx), xoff, dma_dst + (unsigned)(I * NT * 16));
-        else
-            lds_dma16(Y + yload::load_delta(I - NLX, p.ldy), yoff, dma_dst + XBYTES + (unsigned)((I - NLX) * NT * 16));
+        if constexpr (I < NLX) {
+            if constexpr (XK) lds_dma16_at<I * NT * 16, 0>(X, xvo[I], dma_dst);
+            else lds_dma16_at<I * NT * 16, I * (NT / 512) * 128>(X, xvo[0], dma_dst);  // load_delta: 64 rows further along i
+        } else {
+            constexpr int J = I - NLX;
+            if constexpr (YK) lds_dma16_at<XBYTES + J * NT * 16, 0>(Y, yvo[J], dma_dst);
+            else lds_dma16_at<XBYTES + J * NT * 16, J * (NT / 512) * 128>(Y, yvo[0], dma_dst);
+        }
     };
     // Past the end of K the last pair is requested again, into a slot nobody reads any more.
     auto end_request = [&]() {
         next++;
-        wslot = wslot + 1 == NSLOT ? 0 : wslot + 1;
+        woff = woff + SLOT == NSLOT * SLOT ? 0 : woff + SLOT;
         const int kstep = next < NP - 1 ? KGRAN : next == NP - 1 ? KGRAN - tail_skip : 0;
         // (64 leading dimensions fit in 32 bits: the host checks that 256 do)
         X += XK ? kstep : kstep * (int)p.ldx;
         Y += YK ? kstep : kstep * (int)p.ldy;
+    };
+    // FAST pairs: one origin per call, issued behind an MFMA of the compute cluster
+    auto advance_fast = [&](int which) {
+        if (which == 0) X += XK ? KGRAN : KGRAN * (int)p.ldx;
+        else Y += YK ? KGRAN : KGRAN * (int)p.ldy;
     };
 
     // fp16 accumulation: the C operand is requested first, as raw bits that no instruction touches
@@ -830,15 +865,20 @@ void k_gemm_pp64(tiled_params p)
         }
         __builtin_amdgcn_sched_barrier(0);
     };
-    int rslot = 0;
-    auto memory_cluster = [&]() {
-        MIW_LDS const char *xs = lds + rslot * SLOT;
-        begin_request();
+    unsigned roff = 0;  // byte offset in the ring of the slot that is read next
+    // SL: -2: any pair; -1: a FAST pair; >= 0: a FAST pair that reads slot SL, known at compile time (the
+    // loop is unrolled over the ring there: no ring position to keep, and the slot's offset is part of
+    // the instructions' offset fields).  FAST pairs advance the origins in their compute cluster.
+    auto memory_cluster = [&]<int SL>(std::integral_constant<int, SL> sl) {
+        MIW_LDS const char *xs = SL >= 0 ? lds + SL * SLOT : lds + roff;
+        if constexpr (SL >= 0) begin_request_at(sl);
+        else begin_request();
         [&]<int... U>(std::integer_sequence<int, U...>) {
             (cluster_unit(xs, std::integral_constant<int, U>{}), ...);
         }(std::make_integer_sequence<int, NFRAG>{});
-        end_request();
-        rslot = rslot + 1 == NSLOT ? 0 : rslot + 1;
+        if constexpr (SL == -2) end_request();
+        if constexpr (SL == -1) woff = woff + SLOT == NSLOT * SLOT ? 0 : woff + SLOT;
+        if constexpr (SL < 0) roff = roff + SLOT == NSLOT * SLOT ? 0 : roff + SLOT;
         __builtin_amdgcn_sched_barrier(0);
     };
     // ZERO (fp16 accumulation with alpha != 1): the accumulators restart from zero in every slot.
@@ -847,7 +887,14 @@ void k_gemm_pp64(tiled_params p)
     // one after the other and the conversions spread over the whole cluster, the second MFMA of a tile
     // waits for the first and the launch takes 6 to 15 % longer.)
     constexpr int ROUND_LAG = 2;
-    auto compute_cluster = [&]<bool ZERO>(std::bool_constant<ZERO>) {
+    // The tiles whose last MFMA closes the compute cluster would be rounded behind it, with no MFMA to hide
+    // the conversions and the other group waiting at the barrier: the last ROUND_DEFER tiles are rounded
+    // at the end of the wavefront's next memory cluster instead (round_deferred), behind its last
+    // fragment read and before the next compute cluster touches them.  (Measured on 2048^3: 1 or 2 tiles
+    // 3 % faster than none, 3 and more slower again: the memory cluster must stay the shorter one.)
+    constexpr int ROUND_DEFER = F16ACC ? 2 : 0;
+    static_assert(ROUND_DEFER <= NTILE && ROUND_DEFER <= ROUND_LAG, "deferred tiles are the cluster's last");
+    auto compute_cluster = [&]<bool ZERO, bool ADVANCE>(std::bool_constant<ZERO>, std::bool_constant<ADVANCE>) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int h = 0; h < 2; h++)
@@ -860,13 +907,21 @@ void k_gemm_pp64(tiled_params p)
                     else acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fx[h][a], fy[h][b], acc[a][b], 0, 0, 0);
                 }
                 // fp16 accumulation: a tile is rounded ROUND_LAG MFMAs after its last MFMA of the pair
+                if constexpr (ADVANCE)
+                    if (h == 0 && m < 2) advance_fast(m);
                 if constexpr (F16ACC)
-                    if (h == 1 && m >= ROUND_LAG) round_tile(tile_of_mfma(m - ROUND_LAG), std::integral_constant<int, ZERO ? 3 : 1>{});
+                    if (h == 1 && m >= ROUND_LAG && m - ROUND_LAG < NTILE - ROUND_DEFER) round_tile(tile_of_mfma(m - ROUND_LAG), std::integral_constant<int, ZERO ? 3 : 1>{});
                 __builtin_amdgcn_sched_barrier(0);
             }
         if constexpr (F16ACC)
 #pragma unroll
-            for (int m = NTILE > ROUND_LAG ? NTILE - ROUND_LAG : 0; m < NTILE; m++) round_tile(tile_of_mfma(m), std::integral_constant<int, ZERO ? 3 : 1>{});
+            for (int m = NTILE > ROUND_LAG ? NTILE - ROUND_LAG : 0; m < NTILE - ROUND_DEFER; m++) round_tile(tile_of_mfma(m), std::integral_constant<int, ZERO ? 3 : 1>{});
+    };
+    // The first memory cluster rounds sums that are Float16 values already, which changes nothing, and
+    // the last compute cluster's tiles are rounded behind the loop.
+    auto round_deferred = [&]<bool ZERO>(std::bool_constant<ZERO>) {
+#pragma unroll
+        for (int m = NTILE - ROUND_DEFER; m < NTILE; m++) round_tile(tile_of_mfma(m), std::integral_constant<int, ZERO ? 3 : 1>{});
     };
 
     // Folding C (Float32 C laid out as D, alpha == 1): CPT MFMA tiles per cluster over the last
@@ -924,8 +979,12 @@ void k_gemm_pp64(tiled_params p)
         asm volatile("" ::: "memory");
     };
     // RMODE: how the compute cluster rounds its sums (0: fp32 accumulation; 1, 3: see round_tile).
-    auto pair = [&]<int FS, int RMODE>(std::integral_constant<int, FS>, std::integral_constant<int, RMODE>) {
-        memory_cluster();
+    auto pair = [&]<int FS, int RMODE, int SL = -2>(std::integral_constant<int, FS>, std::integral_constant<int, RMODE>, std::integral_constant<int, SL> sl = {}) {
+        memory_cluster(sl);
+        if constexpr (RMODE != 0) {
+            round_deferred(std::bool_constant<RMODE == 3>{});
+            __builtin_amdgcn_sched_barrier(0);
+        }
         if constexpr (FS >= 0) {
             fold_request(std::integral_constant<int, FS>{});
             __builtin_amdgcn_sched_barrier(0);
@@ -950,10 +1009,27 @@ void k_gemm_pp64(tiled_params p)
             wait_loads_and_barrier<(NSLOT - 2) * LPAIR>();
         }
         if constexpr (FS == -2) mask_tail();
-        compute_cluster(std::bool_constant<RMODE == 3>{});
+        compute_cluster(std::bool_constant<RMODE == 3>{}, std::bool_constant<SL != -2>{});
         __builtin_amdgcn_s_barrier();
     };
     constexpr std::integral_constant<int, -1> no_fold{};
+    constexpr std::integral_constant<int, -1> fast_pair{};
+    // NSLOT pairs that need no look at the end of K, the first of which reads slot 0
+#ifdef MIW_PP_TS
+    bool stamp_pair = false;
+#endif
+    auto ring_of_pairs = [&]<int RMODE>(std::integral_constant<int, RMODE> rmode) {
+        [&]<int... S>(std::integer_sequence<int, S...>) {
+            (([&] {
+#ifdef MIW_PP_TS
+                 if constexpr (S == 1)
+                     if (stamp_pair) MIW_PP_STAMP(3)
+#endif
+                 pair(std::integral_constant<int, -1>{}, rmode, std::integral_constant<int, S>{});
+             }()),
+             ...);
+        }(std::make_integer_sequence<int, NSLOT>{});
+    };
     constexpr std::integral_constant<int, -2> last_pair{};
     constexpr std::integral_constant<int, 0> plain{};
 
@@ -961,6 +1037,8 @@ void k_gemm_pp64(tiled_params p)
     if (late_group) __builtin_amdgcn_s_barrier();
     // the loop runs the pairs that neither fold nor are the last one
     const int NPM = fold_c ? NP - NFOLD : NP - 1;
+    // the request of pair pr is pair pr + NSLOT - 1; the pairs before NP - 1 lie a full step apart
+    const int NFAST = min(NPM, max(0, NP - 1 - NSLOT));
     const bool separate_sum = F16ACC && p.alpha != 1.0f;
     if constexpr (F16ACC) {
         // The running sum starts as half(beta * C): with alpha == 1 in the accumulators, which the MFMAs
@@ -968,31 +1046,39 @@ void k_gemm_pp64(tiled_params p)
         constexpr std::integral_constant<int, 1> rolling{};
         constexpr std::integral_constant<int, 3> separate{};
         if (separate_sum) {
-            for (int pr = 0; pr < NPM; pr++) pair(no_fold, separate);
+            int pr = 0;
+            for (; pr + NSLOT <= NFAST; pr += NSLOT) ring_of_pairs(separate);
+            for (; pr < NFAST; pr++) pair(no_fold, separate, fast_pair);
+            next = NSLOT - 1 + pr;
+            for (; pr < NPM; pr++) pair(no_fold, separate);
             pair(last_pair, separate);
+            round_deferred(std::true_type{});
         } else {
 #pragma unroll
             for (int a = 0; a < TI; a++)
 #pragma unroll
                 for (int b = 0; b < TJ; b++) acc[a][b] = cinit[a][b];
-            for (int pr = 0; pr < NPM; pr++) {
-#ifdef MIW_PP_TS
-                if (pr == NPM / 2) MIW_PP_STAMP(2)
-                if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
-#endif
-                pair(no_fold, rolling);
+            int pr = 0;
+            for (; pr + NSLOT <= NFAST; pr += NSLOT) {
+                MIW_PP_MIDDLE(pr)
+                ring_of_pairs(rolling);
             }
+            for (; pr < NFAST; pr++) pair(no_fold, rolling, fast_pair);
+            next = NSLOT - 1 + pr;
+            for (; pr < NPM; pr++) pair(no_fold, rolling);
             MIW_PP_STAMP(9)
             pair(last_pair, rolling);
+            round_deferred(std::false_type{});
         }
     } else {
-        for (int pr = 0; pr < NPM; pr++) {
-#ifdef MIW_PP_TS
-            if (pr == NPM / 2) MIW_PP_STAMP(2)
-            if (pr == NPM / 2 + 1) MIW_PP_STAMP(3)
-#endif
-            pair(no_fold, plain);
+        int pr = 0;
+        for (; pr + NSLOT <= NFAST; pr += NSLOT) {
+            MIW_PP_MIDDLE(pr)
+            ring_of_pairs(plain);
         }
+        for (; pr < NFAST; pr++) pair(no_fold, plain, fast_pair);
+        next = NSLOT - 1 + pr;
+        for (; pr < NPM; pr++) pair(no_fold, plain);
         MIW_PP_STAMP(9)
         if constexpr (CAN_FOLD) {
             if (fold_c) {
