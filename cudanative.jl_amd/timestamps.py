@@ -71,6 +71,10 @@ def main():
     for name, a, b in PHASES:
         x = t[:, :, b] - t[:, :, a]
         print("  %-52s %8.0f %8.0f %8.0f" % (name, np.median(x), x.min(), x.max()))
+    loop = t[:, :, 4] - t[:, :, 1]
+    npairs = (K + 63) // 64
+    print("  whole loop (the pairs that fold C included): %.0f cycles per pair of k-steps at the median (%.0f to %.0f)" % (
+        np.median(loop) / npairs, loop.min() / npairs, loop.max() / npairs))
     cycles = t[:, :, 6] - t[:, :, 0]
     wall = (t[:, :, 7] - t[:, :, 8]) / 100.0
     print("  whole kernel: median %.0f cycles = %.1f us per wavefront (longest %.1f us); %d pairs of k-steps" % (
