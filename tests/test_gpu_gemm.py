@@ -409,6 +409,40 @@ def test_k_tail_every_variant(gpu, orc, al, bl, dl):
             assert np.array_equal(D, orc.gemm_f16acc(g, 64, A, B, C)), (v["name"], al, bl, dl, K)
 
 
+@pytest.mark.parametrize("al,bl", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_pingpong64_every_loop_tier(gpu, orc, al, bl):
+    """The 64-k ping-pong kernels run their K loop in tiers: rings of pairs unrolled over the LDS slots
+    while the request ahead needs no look at the end of K, single pairs of that kind, the pairs that
+    select their step, the pairs that fold C, the last pair.  K from 2 to 15 slots (and one ragged K per
+    length) passes through every combination of them; integers, bit for bit against the oracle, with
+    Float32 accumulation (C folded into the loop where it is Float32 and laid out as D) and, where the
+    variant has it, Float16 accumulation with both roundings (alpha 1 and not)."""
+    served = 0
+    for v in _variants(gpu):
+        if v["pingpong"] and tuple(v["block"][:2]) != (256, 256):
+            bm, bn = v["block"][:2]
+            ran = 0
+            for slots in range(2, 16):
+                for K in (64 * slots, 64 * slots - 16 * (1 + slots % 3)):
+                    g = orc.GemmDesc(M=bm, N=bn, K=K, a_layout=al, b_layout=bl, beta=-1.0)
+                    A, B, C = _inputs(orc, g, 2600 + K + v["id"], ints=True)
+                    D = _run(gpu, orc, g, A, B, C, variant=v["id"])
+                    if D is None:        # (refused, as _run has checked: no rings for these layouts at this tile)
+                        continue
+                    ran += 1
+                    assert np.array_equal(D, orc.gemm(g, A, B, C)), (v["name"], al, bl, K)
+                    if not v["f16_accumulate"] or slots > 8:
+                        continue
+                    for alpha in (1.0, 0.5):
+                        h = orc.GemmDesc(M=bm, N=bn, K=K, a_layout=al, b_layout=bl, c_type=orc.F16, d_type=orc.F16, alpha=alpha)
+                        A, B, C = _inputs(orc, h, 2700 + K + v["id"], ints=True)     # |sums| < 2048: exact in half
+                        D = _run(gpu, orc, h, A, B, C, variant=v["id"], acc_type=F16)
+                        assert np.array_equal(D, orc.gemm_f16acc(h, 64, A, B, C)), (v["name"], al, bl, K, alpha)
+            assert ran in (0, 28), (v["name"], al, bl, ran)      # a layout is served at every K or at none
+            served += ran
+    assert served >= 28
+
+
 def test_k_tail_random_data(gpu, orc):
     """Uniform data, K = 64 q + r on the kernels miw_gemm picks: Float32 accumulation against float64, a
     Float16 D, and Float16 accumulation against the chunked model (chunks of 64, the last one of r)."""
