@@ -443,6 +443,43 @@ def test_pingpong64_every_loop_tier(gpu, orc, al, bl):
     assert served >= 28
 
 
+def test_pingpong64_randomized(gpu, orc):
+    """300 seeded problems on the 64-k ping-pong kernels, forced: extents that the tile does not divide,
+    K from 64 to 1424 in steps of 16, every layout of A, B, C and D, the four C / D type pairs, scalars,
+    batches, with and without C, Float32 and (where the variant has it) Float16 accumulation.  Integers,
+    bit for bit against the oracle."""
+    rng = np.random.default_rng(20)
+    variants = [v for v in _variants(gpu) if v["pingpong"] and tuple(v["block"][:2]) != (256, 256)]
+    assert len(variants) == 3
+    ran = 0
+    for case in range(300):
+        v = variants[case % 3]
+        M, N = 16 * int(rng.integers(16, 48)), 16 * int(rng.integers(16, 48))
+        K = 16 * int(rng.integers(4, 90))
+        al, bl, dl = (int(rng.integers(0, 2)) for _ in range(3))
+        cl = dl if rng.random() < 0.8 else 1 - dl
+        half = bool(v["f16_accumulate"]) and rng.random() < 0.5
+        ct, dt = (orc.F16, orc.F16) if half else (int(rng.integers(0, 2)), int(rng.integers(0, 2)))
+        K = min(K, 640) if half else K          # |sums| stay exact in Float16
+        use_c = int(rng.random() < 0.7)
+        alpha = 1.0 if rng.random() < 0.6 else float(rng.choice([0.5, -2.0]))
+        beta = float(rng.choice([1.0, 0.0, -0.5, 2.0]))
+        g = orc.GemmDesc(M=M, N=N, K=K, a_layout=al, b_layout=bl, c_layout=cl, d_layout=dl, c_type=ct, d_type=dt,
+                         alpha=alpha, beta=beta, use_c=use_c, batch=int(rng.choice([1, 1, 2])))
+        gr = g.resolved()
+        nb = max(gr.batch, 1)
+        A = rng.integers(-2, 3, gr.stride_a * nb).astype(F16)
+        B = rng.integers(-2, 3, gr.stride_b * nb).astype(F16)
+        C = rng.integers(-3, 4, gr.stride_c * nb).astype(orc.np_dtype(ct))
+        D = _run(gpu, orc, g, A, B, C if use_c else None, variant=v["id"], acc_type=F16 if half else F32, prefill=5.0)
+        if D is None:
+            continue
+        ran += 1
+        want = orc.gemm_f16acc(g, 64, A, B, C) if half else orc.gemm(g, A, B, C)
+        assert np.array_equal(D, want), (case, v["name"], M, N, K, al, bl, cl, dl, ct, dt, use_c, alpha, beta, half)
+    assert ran >= 250
+
+
 def test_k_tail_random_data(gpu, orc):
     """Uniform data, K = 64 q + r on the kernels miw_gemm picks: Float32 accumulation against float64, a
     Float16 D, and Float16 accumulation against the chunked model (chunks of 64, the last one of r)."""
